@@ -230,3 +230,128 @@ extern "C" int he_silu_mul(void* out, const void* gate_up, int rows, int I, int 
                            int splits, int dtype, void* stream) {
   return he_gated_act(out, gate_up, rows, I, interleaved, splits, dtype, 1.f, 0.f, 0.f, stream);
 }
+
+// ---- activations and gates of one input -----------------------------------------------------------
+// kind 0: relu(x)^2; 1: gelu with tanh, 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))); 2: silu; 3: relu
+#define HE_ACT_RELU2 0
+#define HE_ACT_GELU_TANH 1
+#define HE_ACT_SILU 2
+#define HE_ACT_RELU 3
+__device__ __forceinline__ float he_unary(float x, int kind) {
+  if (kind == HE_ACT_RELU2) {
+    const float r = fmaxf(x, 0.f);
+    return r * r;
+  }
+  if (kind == HE_ACT_GELU_TANH) return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+  if (kind == HE_ACT_SILU) return x / (1.f + expf(-x));
+  return fmaxf(x, 0.f);
+}
+
+// out[i] = act(x[i]), in place when out == x
+template <typename T>
+__global__ void unary_act_kernel(T* out, const T* x, int64_t n, int kind) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = from_float<T>(he_unary(to_float(x[i]), kind));
+}
+
+extern "C" int he_unary_act(void* out, const void* x, int64_t n, int kind, int dtype, void* stream) {
+  HE_REQUIRE(n >= 0 && kind >= 0 && kind <= 3, "he_unary_act: bad size or kind %d", kind);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_unary_act: unknown dtype %d", dtype);
+  if (n == 0) return 0;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HE_BF16) unary_act_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, n, kind);
+  else unary_act_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)x, n, kind);
+  return he_check_launch("he_unary_act");
+}
+
+// out[r, j] = act(x[r, j]) * table[ids[r], offset + j] for j < W: a gate of the stream's own values on a
+// stretch of a token's row of a second embedding table (row length table_width). A bad id gives zeros.
+template <typename T, typename TT>
+__global__ void token_gate_kernel(T* __restrict__ out, const T* __restrict__ x, const TT* __restrict__ table,
+                                  const int32_t* __restrict__ ids, int rows, int W, int table_width, int offset, int V,
+                                  int kind) {
+  const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)rows * W) return;
+  const int r = (int)(i / W), j = (int)(i % W);
+  const int id = ids[r];
+  float e = 0.f;
+  if (id >= 0 && id < V) e = to_float(table[(int64_t)id * table_width + offset + j]);
+  out[i] = from_float<T>(he_unary(to_float(x[i]), kind) * e);
+}
+
+extern "C" int he_token_gate(void* out, const void* x, const void* table, const void* ids, int rows, int W,
+                             int table_width, int offset, int V, int kind, int dtype, int table_dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && W > 0 && offset >= 0 && offset + W <= table_width && V > 0 && kind >= 0 && kind <= 3,
+             "he_token_gate: bad sizes W=%d offset=%d table_width=%d", W, offset, table_width);
+  HE_REQUIRE((dtype == HE_BF16 || dtype == HE_F32) && (table_dtype == HE_BF16 || table_dtype == HE_F32),
+             "he_token_gate: unknown dtype");
+  if (rows == 0) return 0;
+  const int64_t n = (int64_t)rows * W;
+  const int blocks = (int)((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+#define TG_LAUNCH(T, TT)                                                                                          \
+  token_gate_kernel<T, TT><<<blocks, 256, 0, s>>>((T*)out, (const T*)x, (const TT*)table, (const int32_t*)ids, rows, W, \
+                                                  table_width, offset, V, kind)
+  if (dtype == HE_BF16 && table_dtype == HE_BF16) TG_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == HE_BF16) TG_LAUNCH(bf16_t, float);
+  else if (table_dtype == HE_BF16) TG_LAUNCH(float, bf16_t);
+  else TG_LAUNCH(float, float);
+#undef TG_LAUNCH
+  return he_check_launch("he_token_gate");
+}
+
+// x[r, h * hd + d] *= sigmoid(gate[r * gate_stride + h * vd + d]) * scale for d < vd (the values of a head;
+// its padding up to hd is left as it is): an output gate, element by element, on concatenated heads.
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ x, const T* __restrict__ gate, int64_t gate_stride, int rows, int H,
+                                    int hd, int vd, float scale) {
+  const int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t per = (int64_t)H * vd;
+  if (i >= rows * per) return;
+  const int64_t r = i / per;
+  const int c = (int)(i % per), h = c / vd, d = c % vd;
+  const float g = to_float(gate[r * gate_stride + c]);
+  const int64_t at = r * H * hd + (int64_t)h * hd + d;
+  x[at] = from_float<T>(to_float(x[at]) * scale / (1.f + expf(-g)));
+}
+
+extern "C" int he_sigmoid_gate(void* x, const void* gate, int64_t gate_stride, int rows, int H, int hd, int vd,
+                               float scale, int dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && H > 0 && vd > 0 && hd >= vd && gate_stride >= (int64_t)H * vd, "he_sigmoid_gate: bad sizes");
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_sigmoid_gate: unknown dtype %d", dtype);
+  if (rows == 0) return 0;
+  const int64_t n = (int64_t)rows * H * vd;
+  const int blocks = (int)((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HE_BF16)
+    sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, s>>>((bf16_t*)x, (const bf16_t*)gate, gate_stride, rows, H, hd, vd, scale);
+  else
+    sigmoid_gate_kernel<float><<<blocks, 256, 0, s>>>((float*)x, (const float*)gate, gate_stride, rows, H, hd, vd, scale);
+  return he_check_launch("he_sigmoid_gate");
+}
+
+// out[i] = sa * a[i] + sb * b[i], the sum formed in fp32 (two branches that read the same input, each with its weight)
+template <typename T>
+__global__ void scaled_sum_kernel(T* out, const T* a, const T* b, int64_t n, float sa, float sb) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = from_float<T>(fmaf(sa, to_float(a[i]), sb * to_float(b[i])));
+}
+
+extern "C" int he_scaled_sum(void* out, const void* a, const void* b, int64_t n, float sa, float sb, int dtype,
+                             void* stream) {
+  HE_REQUIRE(n >= 0, "he_scaled_sum: bad size");
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_scaled_sum: unknown dtype %d", dtype);
+  if (n == 0) return 0;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == HE_BF16)
+    scaled_sum_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)a, (const bf16_t*)b, n, sa, sb);
+  else
+    scaled_sum_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)a, (const float*)b, n, sa, sb);
+  return he_check_launch("he_scaled_sum");
+}

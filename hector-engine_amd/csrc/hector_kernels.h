@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 25
+#define HE_ABI_VERSION 26
 
 #ifdef __cplusplus
 extern "C" {
@@ -226,9 +226,25 @@ int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int64_t dt_stri
                 const void* a_log, const void* d_skip, int w_dtype, void* state, int64_t state_stride,
                 int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs,
                 int max_q_len, int R, int Q, int N, int P, int dtype, void* stream);
-// out = rms over each of `parts` stretches of (y * silu(z)) * weight; z[row * z_stride + c].
+// out = rms over each of `parts` stretches of (y * silu(z)) * weight; z[row * z_stride + c]. gate_after 1: out =
+// rms over each stretch of y, * weight * sigmoid(z) * out_scale (the gate behind the norm).
 int he_gated_group_norm(void* out, const void* y_f32, const void* z, int64_t z_stride, const void* weight,
-                        int w_dtype, int rows, int W, int parts, float eps, int dtype, void* stream);
+                        int w_dtype, int rows, int W, int parts, float eps, int gate_after, float out_scale, int dtype,
+                        void* stream);
+
+// ---- a matrix memory carried from token to token (matrix_memory.hip) ---------------------
+// he_mlstm_gates: out_f32 [rows, 2 H] = the logarithms of the input gates (cap tanh((x + b) / cap)) and of the forget
+// gates (logsigmoid of the same bounded number) from their fp32 pre-activations x [rows, 2 H]; cap <= 0: unbounded.
+// he_mlstm_scan: y_f32 [rows, H dv] from q, k [rows, H dk] and v [rows, H dv] (views of rows in_stride elements
+// apart) and the gates' logarithms; S, n and m of a sequence live at state_offset of its row of `state`,
+// he_mlstm_state_floats(H, dk, dv) floats, zeros at a sequence's start. dk up to 512.
+int64_t he_mlstm_state_floats(int H, int dk, int dv);
+int he_mlstm_gates(void* out_f32, const void* x_f32, const void* bias, int bias_dtype, int rows, int H, float cap,
+                   void* stream);
+int he_mlstm_scan(void* y_f32, const void* q, const void* k, const void* v, int64_t in_stride, const void* gates_f32,
+                  void* state, int64_t state_stride, int64_t state_offset, const void* cu_seqlens,
+                  const void* seq_slot, int rows, int num_seqs, int H, int dk, int dv, float q_scale, int dtype,
+                  void* stream);
 
 // ---- routing and head combination (routing.hip) ---------------------------------
 // logits_f32 [rows][E], or null and x [rows][D] (x_dtype) with router_f32 [E][D]: the kernel forms the logits itself.
@@ -279,6 +295,23 @@ int he_apply_penalties_window(void* logits_f32, int rows, int V, int64_t row_str
 int he_sample_rows(void* out_i32, const void* logits_f32, int rows, int V, int64_t row_stride,
                    const void* uniforms_u32, float temperature, int top_k, float top_p,
                    void* stream);
+
+
+// ---- normed branch outputs, activations and gates (norm.hip, elementwise.hip) ---------------------
+// resid += post_weight ? rmsnorm(delta) * post_weight : delta; then out (if given) = next_weight ?
+// rmsnorm(resid) * next_weight : resid, in out_dtype. delta may be null (then only out is made).
+int he_add_normed(void* resid_f32, const void* delta, int delta_dtype, const void* post_weight, float post_eps,
+                  const void* next_weight, float next_eps, int w_dtype, void* out, int out_dtype, int rows, int D,
+                  void* stream);
+// kind: 0 relu^2, 1 gelu (tanh form), 2 silu, 3 relu
+int he_unary_act(void* out, const void* x, int64_t n, int kind, int dtype, void* stream);
+// out[r, j] = act(x[r, j]) * table[ids[r], offset + j], j < W
+int he_token_gate(void* out, const void* x, const void* table, const void* ids, int rows, int W, int table_width,
+                  int offset, int V, int kind, int dtype, int table_dtype, void* stream);
+// x[r, h, d] *= sigmoid(gate[r * gate_stride + h * vd + d]) * scale for d < vd, heads hd apart
+int he_sigmoid_gate(void* x, const void* gate, int64_t gate_stride, int rows, int H, int hd, int vd, float scale,
+                    int dtype, void* stream);
+int he_scaled_sum(void* out, const void* a, const void* b, int64_t n, float sa, float sb, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -369,3 +369,78 @@ extern "C" int he_add_dyt(void* resid_f32, const void* delta, float delta_scale,
 #undef DYT
   return he_check_launch("he_add_dyt");
 }
+
+// ---- a branch output that is normed before it joins the stream ("sandwich" norms) ----------------
+// resid[r, :] += post_w ? delta[r, :] / sqrt(mean(delta[r, :]^2) + post_eps) * post_w : delta[r, :]
+// and then, when out is given,
+// out[r, :] = next_w ? resid[r, :] / sqrt(mean(resid[r, :]^2) + next_eps) * next_w : resid[r, :]
+// (the rows the next reader wants: normed, or the stream itself in the activation dtype). One workgroup a
+// row; the row's new residual values stay in registers between the two sums (D up to PN_EPT * threads).
+#define PN_EPT 16
+template <typename TD, typename TO>
+__global__ void add_normed_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const void* __restrict__ post_w,
+                                  float post_eps, const void* __restrict__ next_w, float next_eps, int w_dtype,
+                                  TO* __restrict__ out, int D) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* r = resid + row * D;
+  const TD* d = delta ? delta + row * D : nullptr;
+  float x[PN_EPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PN_EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    x[e] = (d && i < D) ? to_float(d[i]) : 0.f;
+    ss = fmaf(x[e], x[e], ss);
+  }
+  float inv = 1.f;
+  if (d && post_w) inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)D + post_eps);
+  ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PN_EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < D) {
+      const float g = (d && post_w) ? load_param(post_w, i, w_dtype) : 1.f;
+      x[e] = d ? r[i] + x[e] * inv * g : r[i];
+      if (d) r[i] = x[e];
+    } else {
+      x[e] = 0.f;
+    }
+    ss = fmaf(x[e], x[e], ss);
+  }
+  if (out == nullptr) return;
+  float inv2 = 1.f;
+  if (next_w) inv2 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)D + next_eps);
+  TO* o = out + row * D;
+#pragma unroll
+  for (int e = 0; e < PN_EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < D) o[i] = from_float<TO>(next_w ? x[e] * inv2 * load_param(next_w, i, w_dtype) : x[e]);
+  }
+}
+
+extern "C" int he_add_normed(void* resid_f32, const void* delta, int delta_dtype, const void* post_weight, float post_eps,
+                             const void* next_weight, float next_eps, int w_dtype, void* out, int out_dtype, int rows,
+                             int D, void* stream) {
+  HE_REQUIRE(rows >= 0 && D > 0, "he_add_normed: bad sizes rows=%d D=%d", rows, D);
+  HE_REQUIRE(D <= PN_EPT * 1024, "he_add_normed: width %d above %d", D, PN_EPT * 1024);
+  HE_REQUIRE(w_dtype == HE_F32 || w_dtype == HE_BF16, "he_add_normed: bad weight dtype");
+  HE_REQUIRE((delta == nullptr || delta_dtype == HE_F32 || delta_dtype == HE_BF16) &&
+                 (out == nullptr || out_dtype == HE_F32 || out_dtype == HE_BF16),
+             "he_add_normed: unknown dtype");
+  if (rows == 0) return 0;
+  int threads = 64;
+  while (threads < 1024 && PN_EPT * threads < D) threads <<= 1;
+  while (threads < 256 && 4 * threads < D) threads <<= 1;
+  hipStream_t s = (hipStream_t)stream;
+#define PN_LAUNCH(TD, TO)                                                                                        \
+  add_normed_kernel<TD, TO><<<rows, threads, 0, s>>>((float*)resid_f32, (const TD*)delta, post_weight, post_eps, \
+                                                     next_weight, next_eps, w_dtype, (TO*)out, D)
+  const bool db = delta != nullptr && delta_dtype == HE_BF16, ob = out != nullptr && out_dtype == HE_BF16;
+  if (db && ob) PN_LAUNCH(bf16_t, bf16_t);
+  else if (db) PN_LAUNCH(bf16_t, float);
+  else if (ob) PN_LAUNCH(float, bf16_t);
+  else PN_LAUNCH(float, float);
+#undef PN_LAUNCH
+  return he_check_launch("he_add_normed");
+}

@@ -348,32 +348,42 @@ extern "C" int he_ssm_scan(void* y_f32, const void* xbc, const void* dt_in, int6
 }
 
 // ---- gated, grouped RMS norm ------------------------------------------------------------------
-// out[row, c] = v / sqrt(mean over c's part of v^2 + eps) * weight[c], v = y[row, c] * silu(z[row, c]):
+// gate_after 0:  out[row, c] = v / sqrt(mean over c's part of v^2 + eps) * weight[c], v = y[row, c] * silu(z[row, c]):
 // the product with silu(z) is formed first and normalised afterwards, each of the `parts` equal stretches of
-// a row by a root mean square of its own. One workgroup a (row, part).
+// a row by a root mean square of its own.
+// gate_after 1:  out[row, c] = y / sqrt(mean over c's part of y^2 + eps) * weight[c] * sigmoid(z[row, c]) * out_scale:
+// the stretch is normalised as it is and the gate, a sigmoid, multiplies the result. One workgroup a (row, part).
 template <typename T>
 __global__ void gated_group_norm_kernel(T* __restrict__ out, const float* __restrict__ y, const T* __restrict__ z,
                                         int64_t z_stride, const void* __restrict__ weight, int w_dtype, int W,
-                                        int parts, float eps) {
+                                        int parts, float eps, int gate_after, float out_scale) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.y;
   const int width = W / parts;
   const int c0 = blockIdx.x * width;
   float sq = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = y[row * W + c0 + i] * ss_silu(to_float(z[row * z_stride + c0 + i]));
+    float v = y[row * W + c0 + i];
+    if (!gate_after) v *= ss_silu(to_float(z[row * z_stride + c0 + i]));
     sq = fmaf(v, v, sq);
   }
   const float total = block_sum(sq, scratch);
   const float inv = 1.f / sqrtf(total / (float)width + eps);
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float v = y[row * W + c0 + i] * ss_silu(to_float(z[row * z_stride + c0 + i]));
-    out[row * W + c0 + i] = from_float<T>(v * inv * load_param(weight, c0 + i, w_dtype));
+    const float g = to_float(z[row * z_stride + c0 + i]);
+    float v = y[row * W + c0 + i];
+    if (!gate_after) {
+      v = v * ss_silu(g) * inv * load_param(weight, c0 + i, w_dtype);
+    } else {
+      v = v * inv * load_param(weight, c0 + i, w_dtype) * (out_scale / (1.f + expf(-g)));
+    }
+    out[row * W + c0 + i] = from_float<T>(v);
   }
 }
 
 extern "C" int he_gated_group_norm(void* out, const void* y_f32, const void* z, int64_t z_stride, const void* weight,
-                                   int w_dtype, int rows, int W, int parts, float eps, int dtype, void* stream) {
+                                   int w_dtype, int rows, int W, int parts, float eps, int gate_after, float out_scale,
+                                   int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && W > 0 && parts > 0 && W % parts == 0, "he_gated_group_norm: bad sizes W=%d parts=%d", W, parts);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_gated_group_norm: unknown dtype %d", dtype);
   if (rows == 0) return 0;
@@ -383,9 +393,9 @@ extern "C" int he_gated_group_norm(void* out, const void* y_f32, const void* z, 
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HE_BF16)
     gated_group_norm_kernel<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)out, (const float*)y_f32, (const bf16_t*)z, z_stride,
-                                                             weight, w_dtype, W, parts, eps);
+                                                             weight, w_dtype, W, parts, eps, gate_after, out_scale);
   else
     gated_group_norm_kernel<float><<<grid, threads, 0, s>>>((float*)out, (const float*)y_f32, (const float*)z, z_stride,
-                                                            weight, w_dtype, W, parts, eps);
+                                                            weight, w_dtype, W, parts, eps, gate_after, out_scale);
   return he_check_launch("he_gated_group_norm");
 }

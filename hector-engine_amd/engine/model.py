@@ -84,6 +84,7 @@ class DecoderModel:
         """ids: int32 [rows]. Returns fp32 logits [n_want, vocab] of the rows
         named by want_rows (int32 [n_want]), or None when nothing is wanted."""
         rows = ctx.rows
+        ctx.tokens = ids
         resid = self.embedding.forward(ids, rows, ctx)
         stream = ResidualStream(resid, rows)
         embedded = None

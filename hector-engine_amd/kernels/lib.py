@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 25
+EXPECTED_ABI = 26
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -61,7 +61,17 @@ _SIGNATURES = {
     "he_ssm_state_floats": [c_int, c_int, c_int],
     "he_ssm_scan": [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_i64, c_i64, c_ptr, c_ptr,
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
-    "he_gated_group_norm": [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_gated_group_norm": [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_int, c_int, c_int, c_int, c_f32, c_int, c_f32,
+                            c_int, c_ptr],
+    "he_mlstm_state_floats": [c_int, c_int, c_int],
+    "he_mlstm_gates": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_ptr],
+    "he_mlstm_scan": [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_int, c_int,
+                      c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_add_normed": [c_ptr, c_ptr, c_int, c_ptr, c_f32, c_ptr, c_f32, c_int, c_ptr, c_int, c_int, c_int, c_ptr],
+    "he_unary_act": [c_ptr, c_ptr, c_i64, c_int, c_int, c_ptr],
+    "he_token_gate": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_sigmoid_gate": [c_ptr, c_ptr, c_i64, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_scaled_sum": [c_ptr, c_ptr, c_ptr, c_i64, c_f32, c_f32, c_int, c_ptr],
     "he_route_tokens": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_int, c_int, c_int, c_int,
                         c_int, c_int, c_int, c_f32, c_ptr],
     "he_routed_act": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_ptr],
@@ -99,6 +109,7 @@ _SIGNATURES = {
 _RESTYPES = {
     "he_attention_plain_workspace_floats": c_i64,
     "he_ssm_state_floats": c_i64,
+    "he_mlstm_state_floats": c_i64,
     "he_gemm_plain_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
     "he_attention_decode_fused_workspace_floats": c_i64,

@@ -615,9 +615,12 @@ def ssm_scan(y, xbc, dt, dt_bias, a_log, d_skip, state, state_offset: int, cu_se
 
 
 @_op("gated_group_norm")
-def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float) -> None:
+def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float, gate_after: bool = False,
+                     out_scale: float = 1.0) -> None:
     """out[rows, W] = (y * silu(z)), each of `parts` equal stretches of a row divided by its own root mean
-    square, times weight. y fp32 [rows, W]; z a view [rows, W] of wider rows in out's dtype."""
+    square, times weight. y fp32 [rows, W]; z a view [rows, W] of wider rows in out's dtype. gate_after: each
+    stretch of y is divided by its own root mean square as it is, and the result is multiplied by weight,
+    sigmoid(z) and out_scale."""
     W = weight.shape[0]
     _need(out, "out", None, (None, W))
     _need(y, "y", torch.float32, (None, W))
@@ -628,8 +631,142 @@ def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float) -> No
         raise ValueError("gated_group_norm: buffers smaller than the row count, or parts that do not divide the width")
     L = _lib.load()
     _lib.check(L.he_gated_group_norm(out.data_ptr(), y.data_ptr(), z.data_ptr(), z.stride(0), weight.data_ptr(),
-                                     dtype_code(weight.dtype), rows, W, parts, float(eps), dtype_code(out.dtype),
-                                     _stream()))
+                                     dtype_code(weight.dtype), rows, W, parts, float(eps), int(gate_after),
+                                     float(out_scale), dtype_code(out.dtype), _stream()))
+
+
+ACT_KINDS = {"relu2": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
+
+
+@_op("add_normed")
+def add_normed(resid_f32, delta, post_weight, post_eps: float, next_weight, next_eps: float, out, rows: int) -> None:
+    """resid += rmsnorm(delta) * post_weight (post_weight None: += delta; delta None: nothing is added); then,
+    with out, out = rmsnorm(resid) * next_weight (next_weight None: out = resid in out's dtype)."""
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    if resid_f32.numel() < rows * D:
+        raise ValueError("add_normed: resid smaller than the row count")
+    w_dtype = None
+    for name, w in (("post_weight", post_weight), ("next_weight", next_weight)):
+        if w is not None:
+            _need(w, name, w_dtype, (D,))
+            w_dtype = w.dtype
+    for name, t in (("delta", delta), ("out", out)):
+        if t is not None:
+            _need(t, name)
+            if t.shape[-1] != D or t.numel() < rows * D:
+                raise ValueError(f"add_normed: {name} does not match [rows, {D}]")
+    L = _lib.load()
+    _lib.check(L.he_add_normed(resid_f32.data_ptr(), _ptr(delta), dtype_code(delta.dtype) if delta is not None else F32,
+                               _ptr(post_weight), float(post_eps), _ptr(next_weight), float(next_eps),
+                               dtype_code(w_dtype) if w_dtype is not None else F32, _ptr(out),
+                               dtype_code(out.dtype) if out is not None else F32, rows, D, _stream()))
+
+
+@_op("unary_act")
+def unary_act(out, x, rows: int, kind: str) -> None:
+    """out[rows, W] = act(x[rows, W]); kind: relu2, gelu_tanh, silu, relu. In place when out is x."""
+    _need(out, "out", x.dtype)
+    _need(x, "x")
+    W = x.shape[-1]
+    if out.shape[-1] != W or min(out.numel(), x.numel()) < rows * W:
+        raise ValueError("unary_act: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_unary_act(out.data_ptr(), x.data_ptr(), rows * W, ACT_KINDS[kind], dtype_code(x.dtype), _stream()))
+
+
+@_op("token_gate")
+def token_gate(out, x, table, ids, rows: int, offset: int, kind: str) -> None:
+    """out[r, j] = act(x[r, j]) * table[ids[r], offset + j] for the W columns of x."""
+    _need(x, "x")
+    W = x.shape[-1]
+    _need(out, "out", x.dtype, (None, W))
+    _need(table, "table")
+    _need(ids, "ids", torch.int32)
+    if table.dim() != 2 or offset < 0 or offset + W > table.shape[1]:
+        raise ValueError("token_gate: the stretch does not lie inside a row of the table")
+    if min(out.shape[0], x.shape[0], ids.numel()) < rows:
+        raise ValueError("token_gate: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_token_gate(out.data_ptr(), x.data_ptr(), table.data_ptr(), ids.data_ptr(), rows, W, table.shape[1],
+                               offset, table.shape[0], ACT_KINDS[kind], dtype_code(x.dtype), dtype_code(table.dtype),
+                               _stream()))
+
+
+@_op("sigmoid_gate")
+def sigmoid_gate(x, gate, rows: int, H: int, hd: int, vd: int, scale: float = 1.0) -> None:
+    """x[r, h, d] *= sigmoid(gate[r, h * vd + d]) * scale for d < vd; x [rows, H * hd], gate a view [rows, H * vd]
+    of wider rows."""
+    _need(x, "x", None, (None, H * hd))
+    if gate.dtype != x.dtype or gate.dim() != 2 or gate.shape[1] != H * vd or gate.stride(1) != 1:
+        raise ValueError("sigmoid_gate: gate must be a [rows, H * vd] view in x's dtype")
+    if min(x.shape[0], gate.shape[0]) < rows or hd < vd:
+        raise ValueError("sigmoid_gate: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_sigmoid_gate(x.data_ptr(), gate.data_ptr(), gate.stride(0), rows, H, hd, vd, float(scale),
+                                 dtype_code(x.dtype), _stream()))
+
+
+@_op("scaled_sum")
+def scaled_sum(out, a, b, rows: int, sa: float, sb: float) -> None:
+    """out = sa * a + sb * b over [rows, D]."""
+    _need(a, "a")
+    D = a.shape[-1]
+    _need(b, "b", a.dtype, (None, D))
+    _need(out, "out", a.dtype, (None, D))
+    if min(out.shape[0], a.shape[0], b.shape[0]) < rows:
+        raise ValueError("scaled_sum: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_scaled_sum(out.data_ptr(), a.data_ptr(), b.data_ptr(), rows * D, float(sa), float(sb),
+                               dtype_code(a.dtype), _stream()))
+
+
+def mlstm_state_floats(H: int, dk: int, dv: int) -> int:
+    """Floats of a sequence's matrix memory (S with padded key dims, and n and m once a workgroup)."""
+    return int(_lib.load().he_mlstm_state_floats(H, dk, dv))
+
+
+@_op("mlstm_gates")
+def mlstm_gates(out, x, bias, rows: int, H: int, cap: float) -> None:
+    """out fp32 [rows, 2 H] = the logarithms of the input gates and of the forget gates from x fp32 [rows, 2 H]."""
+    _need(out, "out", torch.float32, (None, 2 * H))
+    _need(x, "x", torch.float32, (None, 2 * H))
+    if bias is not None:
+        _need(bias, "bias", None, (2 * H,))
+    if min(out.shape[0], x.shape[0]) < rows:
+        raise ValueError("mlstm_gates: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_mlstm_gates(out.data_ptr(), x.data_ptr(), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
+                                rows, H, float(cap), _stream()))
+
+
+@_op("mlstm_scan")
+def mlstm_scan(y, q, k, v, gates, state, state_offset: int, cu_seqlens, seq_slot, rows: int, num_seqs: int,
+               H: int, dk: int, dv: int, q_scale: float) -> None:
+    """y (fp32 [rows, H dv]) = the matrix memory's answers to q, after each row's k and v went in under the
+    row's gates (gates: fp32 [rows, 2 H], the logarithms). q, k [rows, H dk] and v [rows, H dv] are views of
+    the same wider rows; the memory lives at byte state_offset of a sequence's row of `state` and is carried on."""
+    _need(y, "y", torch.float32, (None, H * dv))
+    _need(gates, "gates", torch.float32, (None, 2 * H))
+    stride = q.stride(0)
+    for name, t, w in (("q", q, H * dk), ("k", k, H * dk), ("v", v, H * dv)):
+        if t.dtype != q.dtype or t.dim() != 2 or t.shape[1] != w or t.stride(1) != 1 or t.stride(0) != stride \
+                or t.shape[0] < rows:
+            raise ValueError(f"mlstm_scan: {name} must be a [rows, {w}] view of the rows q lies in")
+    if y.shape[0] < rows or gates.shape[0] < rows:
+        raise ValueError("mlstm_scan: buffers smaller than the row count")
+    if state.dtype != torch.uint8 or state.dim() != 2 or state.stride(1) != 1 \
+            or state.shape[1] < state_offset + 4 * mlstm_state_floats(H, dk, dv):
+        raise ValueError("mlstm_scan: state must be uint8 [slots, bytes] with room for the memory")
+    _need(cu_seqlens, "cu_seqlens", torch.int32)
+    _need(seq_slot, "seq_slot", torch.int32)
+    if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs:
+        raise ValueError("mlstm_scan: metadata shorter than the step")
+    L = _lib.load()
+    _lib.check(L.he_mlstm_scan(y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, gates.data_ptr(),
+                               state.data_ptr(), state.stride(0), state_offset, cu_seqlens.data_ptr(),
+                               seq_slot.data_ptr(), rows, num_seqs, H, dk, dv, float(q_scale), dtype_code(q.dtype),
+                               _stream()))
 
 
 @_op("route_tokens")

@@ -19,8 +19,15 @@ Options of the same part, each off unless its parameter says otherwise:
               counted from position 0 of the sequence.
   sinks       a stored number per head joins the softmax's denominator as exp(sink_h); it has no
               key and no value, is not scaled and counts once.
+  sink_value  a constant in place of the stored sinks: every head's softmax has exp(sink_value) more in its
+              denominator (0.0: one is added), and no tensor is read.
   head_gate   head h's output is multiplied by sigmoid(g_h), g = Wg n with one row of Wg a head;
               the rows of Wg ride behind q||k||v in the one product.
+  out_gate    the concatenated heads are multiplied element by element by sigmoid(Wg n), Wg with a row for
+              every value of every head (tensor `gate`); its rows ride behind q||k||v likewise.
+  qk_norm     "projection": q (all heads' rows of a token at once) is divided by its root mean square
+              (eps `qk_norm_eps`) and multiplied by a stored vector of that size, k likewise; after the
+              bias and before the position encoding.
   q_temp      {coef, every}: the q of position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
   score_maps  2: differential attention. A head has two queries and a kv head two keys (in the q and k
               matrices a head's rows for map 1 stand in front of its rows for map 2); the two maps are
@@ -31,7 +38,7 @@ Options of the same part, each off unless its parameter says otherwise:
               so that the heads of one (kv head, map) are neighbours, and the value rows of a kv head
               stand once for each of its maps; ops.diff_heads then joins the pairs.
   names       the suffixes of its tensors (q, k, v, o, q_bias, k_bias, v_bias, o_bias, sinks, gate,
-              lq1, lk1, lq2, lk2).
+              lq1, lk1, lq2, lk2, q_norm, k_norm).
 """
 from __future__ import annotations
 
@@ -47,7 +54,7 @@ from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, Ste
 _NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
           "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
           "sinks": "sinks", "gate": "gate.weight", "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2",
-          "lk2": "lambda_k2"}
+          "lk2": "lambda_k2", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
 from .linear import Linear
 
 
@@ -89,14 +96,25 @@ class Attention(Mixer):
         self.chunk = param(params, "chunk", int, 0)
         self.has_sinks = param(params, "sinks", bool, False)
         self.head_gate = param(params, "head_gate", bool, False)
+        self.out_gate = param(params, "out_gate", bool, False)
+        self.sink_value = param(params, "sink_value", float, None)
+        self.qk_norm = param(params, "qk_norm", str, "")
+        self.qk_norm_eps = param(params, "qk_norm_eps", float, 1e-6)
+        self.q_norm_w = self.k_norm_w = None
         self.maps = param(params, "score_maps", int, 1)
         self.diff = param(params, "diff", float, 0.0)
         self.diff_eps = param(params, "diff_eps", float, 1e-6)
         self.lam = 0.0                      # lambda of a differential attention, from its four vectors (bind)
         qt = param(params, "q_temp", dict, None)
         self.q_temp = None if not qt else (float(qt["coef"]), int(qt["every"]))
-        if self.maps not in (1, 2) or (self.maps == 2 and self.head_gate):
-            raise ValueError(f"attention: score_maps {self.maps} must be 1 or 2 (and 2 goes without head gates)")
+        if self.maps not in (1, 2) or (self.maps == 2 and (self.head_gate or self.out_gate or self.qk_norm)):
+            raise ValueError(f"attention: score_maps {self.maps} must be 1 or 2 (and 2 goes without gates and q/k norms)")
+        if self.head_gate and self.out_gate:
+            raise ValueError("attention: head_gate and out_gate exclude each other")
+        if self.qk_norm not in ("", "projection"):
+            raise ValueError(f"attention: unknown qk_norm '{self.qk_norm}'")
+        if self.has_sinks and self.sink_value is not None:
+            raise ValueError("attention: stored sinks and sink_value exclude each other")
         if self.q_temp is not None and self.q_temp[1] <= 0:
             raise ValueError(f"attention: q_temp.every {self.q_temp[1]} must be positive")
         # the heads as the kernels count them: a differential head is two, one a score map
@@ -122,7 +140,10 @@ class Attention(Mixer):
         self._chosen_version = -1
         self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0   # else the plain kernel
         # what the fused one-token kernel and the kernels without these options do not take
-        self.extras = self.chunk > 0 or self.has_sinks or self.head_gate or self.maps > 1 or self.q_temp is not None
+        self.extras = self.chunk > 0 or self.has_sinks or self.head_gate or self.maps > 1 or self.q_temp is not None \
+            or self.out_gate or self.sink_value is not None or bool(self.qk_norm)
+        # rows of the gate's matrix behind q||k||v: one a head, or one for every value of every head
+        self.gate_rows = self.H if self.head_gate else self.H * self.vd if self.out_gate else 0
 
     def children(self):
         return [self.position]
@@ -151,8 +172,12 @@ class Attention(Mixer):
             specs[n["o_bias"]] = TensorSpec((self.hidden,))
         if self.has_sinks:
             specs[n["sinks"]] = TensorSpec((self.H,), ("normal", 1.0))
-        if self.head_gate:
-            specs[n["gate"]] = TensorSpec((self.H, self.hidden))
+        if self.gate_rows:
+            specs[n["gate"]] = TensorSpec((self.gate_rows, self.hidden))
+        if self.qk_norm:
+            specs[n["q_norm"]] = TensorSpec((self.H * hd,), ("gain", 1.0, 0.1))
+            if self.kv_projection:
+                specs[n["k_norm"]] = TensorSpec((self.KVH * hd,), ("gain", 1.0, 0.1))
         specs.update(self.position.tensor_specs())
         return specs
 
@@ -160,7 +185,7 @@ class Attention(Mixer):
         p, n = self.prefix, self._names
         names = ["q"] + (["k", "v"] if self.kv_projection else [])
         ws = [self._by_map(x, tensors.pop(n[x])) for x in names]
-        gate_w = tensors.pop(n["gate"]) if self.head_gate else None
+        gate_w = tensors.pop(n["gate"]) if self.gate_rows else None
         if gate_w is not None:
             ws.append(gate_w)          # the gate's rows ride behind q||k||v: one product
             spare = -sum(w.shape[0] for w in ws) % 8
@@ -184,10 +209,10 @@ class Attention(Mixer):
         self.qkv = Linear(w, bias_for(b, w.shape[0]))
         q_rows = self.Hk * self.hd
         if gate_w is not None and self.kv_projection:
-            spare = -(q_rows + self.H) % 8
+            spare = -(q_rows + self.gate_rows) % 8
             self.q_only = Linear(torch.cat([ws[0], gate_w, torch.zeros((spare, gate_w.shape[1]), dtype=gate_w.dtype,
                                                                        device=gate_w.device)], 0).contiguous(),
-                                 None if b is None else bias_for(b[:q_rows], q_rows + self.H + spare))
+                                 None if b is None else bias_for(b[:q_rows], q_rows + self.gate_rows + spare))
         else:
             self.q_only = Linear(w if gate_w is not None else w[:q_rows],
                                  None if b is None else bias_for(b[:q_rows], w.shape[0] if gate_w is not None else q_rows))
@@ -204,6 +229,11 @@ class Attention(Mixer):
         self.o_proj = Linear(wo, tensors.get(n["o_bias"]))
         if self.has_sinks:
             self.sinks = tensors[n["sinks"]]
+        elif self.sink_value is not None:
+            self.sinks = torch.full((self.H,), self.sink_value, dtype=torch.float32, device=wo.device)
+        if self.qk_norm:
+            self.q_norm_w = tensors[n["q_norm"]]
+            self.k_norm_w = tensors[n["k_norm"]] if self.kv_projection else None
         self.position.bind(tensors)
 
     def _by_map(self, which: str, t: torch.Tensor) -> torch.Tensor:
@@ -219,7 +249,7 @@ class Attention(Mixer):
         return t.reshape(self.KVH, 1, self.vd, *rest).expand(self.KVH, 2, self.vd, *rest).reshape(
             2 * t.shape[0], *rest).contiguous()
 
-    def _project(self, out, rows: int, ctx: StepContext):
+    def _project(self, out, rows: int, ctx: StepContext, gate=None):
         """The output product behind the attention kernels (a differential attention joins its pairs
         of heads first)."""
         if self.maps == 2:
@@ -227,6 +257,8 @@ class Attention(Mixer):
             ops.diff_heads(mixed, out, rows, self.H, self.KVH, self.pd, self.vd, self.lam, 1.0 - self.diff,
                            self.diff_eps)
             out = mixed
+        if self.out_gate:
+            ops.sigmoid_gate(out, gate, rows, self.H, self.pd, self.vd)
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
 
     def forward(self, x, ctx: StepContext, cache: LayerCache):
@@ -283,8 +315,15 @@ class Attention(Mixer):
         rot = self.position.rotary()
         # With a rotation (or no encoding) the bias is added inside the fused kernel;
         # any other encoding sees q and k with their bias already added.
-        fused_bias = not self.position.custom
+        fused_bias = not self.position.custom and not self.qk_norm
         qkv = proj(x, rows, ctx, use_bias=not fused_bias)
+        if self.qk_norm:
+            # each token's q (all heads at once), and its k, by a root mean square of their own, in place
+            wide = qkv.stride(0)
+            ops.rmsnorm_rows(qkv, qkv, self.q_norm_w, rows, H * hd, wide, wide, self.qk_norm_eps)
+            if writes:
+                kq = qkv.reshape(-1)[H * hd:]       # the same rows, begun at their k columns
+                ops.rmsnorm_rows(kq, kq, self.k_norm_w, rows, KVH * hd, wide, wide, self.qk_norm_eps)
         if not fused_bias:
             q_cols, kv_cols = H * hd, KVH * hd
             qv = qkv[:, :q_cols].unflatten(1, (H, hd))
@@ -298,9 +337,9 @@ class Attention(Mixer):
                            key_dim=hd, value_dim=self.vd, interleaved=self.position.interleaved,
                            mscale=self.position.mscale, q_temp=self.q_temp)
         gate = None
-        if self.head_gate:
+        if self.gate_rows:
             at = H * hd + (KVH * (hd + self.vd) if writes else 0)
-            gate = qkv[:rows, at:at + H]
+            gate = qkv[:rows, at:at + self.gate_rows]
         return q, gate
 
     def _run_plain(self, x, ctx: StepContext, cache: LayerCache):
@@ -312,8 +351,8 @@ class Attention(Mixer):
         ws = ctx.alloc((floats,), torch.float32) if floats else None
         ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                             ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                            self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self._project(out, rows, ctx)
+                            self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+        return self._project(out, rows, ctx, gate)
 
     def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):
         """One-token steps of the head sizes and encodings the fused kernel does not take."""
@@ -324,8 +363,8 @@ class Attention(Mixer):
         ws = ctx.alloc((max(floats, 1),), torch.float32)
         ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                              ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                             self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self._project(out, rows, ctx)
+                             self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+        return self._project(out, rows, ctx, gate)
 
     def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
         """Prompt steps and mixed steps."""
@@ -348,8 +387,8 @@ class Attention(Mixer):
         ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                               ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                               rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws,
-                              chunk=self.chunk, sinks=self.sinks, gate=gate)
-        return self._project(out, rows, ctx)
+                              chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+        return self._project(out, rows, ctx, gate)
 
 
 _BF16 = (torch.bfloat16,)

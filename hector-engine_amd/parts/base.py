@@ -160,6 +160,8 @@ class StepContext:
                                           # rows of the step's rows, gathered by the host into the step's metadata
                                           # (one-token steps that replay a graph; a mixer may read it in place of
                                           # LayerCache.page_table[seq_slot[row_seq[row]]] and skip that chain)
+        self.tokens = None                # int32 [rows] the step's token ids (set by the model; a part that looks a token
+                                          # up in a table of its own reads them)
         self.next_norm = None             # the norm that reads the stream after the running block (set by the model)
         self.sink = None                  # ResidualSink offered to the running mixer / feed-forward
 
@@ -280,6 +282,18 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class TokenInput(Part):
+    """A contribution to the stream that depends on the row's token itself as well as on the stream:
+    forward(x, ctx) takes the stream's rows in the activation dtype and ctx.tokens and returns [rows, D];
+    post_norm() is (gain, eps) of the RMS norm its result passes before it joins the stream, or None."""
+
+    def post_norm(self) -> tuple | None:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block(Part):
     """Arrangement of a layer's parts around the residual stream."""
 
@@ -352,13 +366,14 @@ class ResidualStream:
         self.pending: torch.Tensor | None = None
         self.pending_scale = 1.0                               # the stream gains pending_scale * pending
         self.prepared: tuple[Norm, NormedRows] | None = None   # rows already made for that norm
+        self.ready: tuple[Norm, torch.Tensor] | None = None    # that norm of the stream as it stands, already computed
 
     def add(self, delta, ctx: StepContext, scale: float = 1.0) -> None:
         """The stream gains scale * delta. delta: a tensor [rows, D], or None when the producer
         has added its result through a ResidualSink."""
         if delta is None:
             return
-        self.prepared = None
+        self.prepared = self.ready = None
         if self.pending is not None:
             self.materialize(ctx)
         self.pending = delta
@@ -378,6 +393,9 @@ class ResidualStream:
         """norm(resid + pending) in the activation dtype. With rows_ok the caller takes
         NormedRows too (rows a product has left for this norm)."""
         prepared, self.prepared = self.prepared, None
+        ready, self.ready = self.ready, None
+        if ready is not None and ready[0] is norm and self.pending is None:
+            return ready[1]
         if prepared is not None and prepared[0] is norm and self.pending is None:
             return prepared[1] if rows_ok else prepared[1].tensor(ctx)
         if self.pending is not None and self.pending_scale != 1.0:
@@ -399,7 +417,7 @@ class ResidualStream:
 # registries
 # ----------------------------------------------------------------------------
 
-CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head")
+CATEGORIES = ("mixer", "feed_forward", "norm", "position", "block", "embedding", "head", "token_input")
 _registries: dict[str, dict[str, Callable[..., Part]]] = {c: {} for c in CATEGORIES}
 
 

@@ -93,3 +93,51 @@ class GatedMLP(FeedForward):
             self.down(h, n, ctx, out=out[r0:r0 + n])
             ctx.scratch.release(turn)       # the next turn reuses h and gate||up
         return out
+
+
+@register_part("feed_forward", "dense_mlp")
+class DenseMLP(FeedForward):
+    """Feed-forward without a gate: d = act(x Wu^T) Wd^T, no biases. activation: "relu2" (the square of
+    relu), "gelu_tanh", "silu" or "relu". names: the suffixes of its tensors (up, down)."""
+
+    accepts_normed_rows = True
+
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        self.hidden = param(params, "hidden_size", int)
+        self.inter = param(params, "intermediate_size", int)
+        self.act = param(params, "activation", str, "relu2")
+        if self.act not in ops.ACT_KINDS:
+            raise ValueError(f"dense_mlp: unsupported activation '{self.act}', have {sorted(ops.ACT_KINDS)}")
+        names = param(params, "names", dict, {})
+        self._names = {k: tensor_name(prefix, names, k, d) for k, d in
+                       (("up", "up_proj.weight"), ("down", "down_proj.weight"))}
+        self.up: Linear | None = None
+        self.down: Linear | None = None
+
+    def tensor_specs(self):
+        n = self._names
+        return {n["up"]: TensorSpec((self.inter, self.hidden)), n["down"]: TensorSpec((self.hidden, self.inter))}
+
+    def bind(self, tensors):
+        n = self._names
+        self.up = Linear(tensors[n["up"]])
+        self.down = Linear(tensors[n["down"]])
+
+    def forward(self, x, ctx: StepContext):
+        rows = ctx.rows
+        if rows <= _ROW_CHUNK:
+            h = self.up(x, rows, ctx)
+            ops.unary_act(h, h, rows, self.act)
+            return self.down(h, rows, ctx, sink=ctx.take_sink())
+        if not isinstance(x, torch.Tensor):
+            x = x.tensor(ctx)
+        out = ctx.alloc((rows, self.hidden))
+        for r0 in range(0, rows, _ROW_CHUNK):
+            n = min(_ROW_CHUNK, rows - r0)
+            turn = ctx.scratch.mark()
+            h = self.up(x[r0:r0 + n], n, ctx)
+            ops.unary_act(h, h, n, self.act)
+            self.down(h, n, ctx, out=out[r0:r0 + n])
+            ctx.scratch.release(turn)
+        return out
