@@ -4,7 +4,7 @@ token ids) on one MI355X, with prefill and roofline figures on the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
                     [--context C] [--prompt P]
-    python bench.py --design volonex | penasun      (another measurement: see below)
+    python bench.py --design volonex | penasun | butolorn      (another measurement: see below)
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
@@ -28,7 +28,8 @@ the machine runs every kernel of the one-token step 4 to 6 % slower than afterwa
 leaves its first run and its thermal-low samples out: OPTIMIZATION_NOTES.md:114-117); `repeats` holds
 every timed run, the earlier ones still show it.
 
---design volonex (or penasun) leaves the run above aside and measures that design beside Qwen2 at equal layer
+--design volonex (or penasun; butolorn is measured beside Penasun, the other design whose layers carry a state
+of fixed size) leaves the run above aside and measures that design beside Qwen2 at equal layer
 sizes (random weights, bf16, four layers of each of a few sizes that resemble real models' layers): prompt
 tokens a second for one prompt of 2,048 tokens, decoded tokens a second at batch 8 and batch 1 behind such
 prompts, and, from a second pass with an event pair around every launch, the mean time of each kind of
@@ -139,6 +140,25 @@ def penasun_configs(sz):
     return qwen, config_from_dict(penasun)
 
 
+def butolorn_configs(sz):
+    """(Penasun configuration, Butolorn configuration) of one set of layer sizes. Penasun is the design beside it:
+    both alternate a layer that carries a state of fixed size per sequence with an attention layer. The Butolorn
+    layers are, in turn, an attention and a matrix memory side by side (the attention as wide as the Qwen2 layer's,
+    the memory with heads of 128 key and 256 value dims, as many as make its values as wide as the model) and an
+    attention alone, each with a dense feed-forward of the Qwen2 layer's width and a token input of 64 columns."""
+    from hector_engine_amd.registry import config_from_dict
+    _, penasun = penasun_configs(sz)
+    rot = dict(base=1000000.0, dims=sz["dim"] // 2)
+    attention = dict(heads=sz["heads"], kv_heads=sz["kv_heads"], dim=sz["dim"], vdim=sz["vdim"], scale=sz["dim"] ** -0.5, rot=rot)
+    pair = dict(left=attention, left_scale=1.0, right_scale=1.0,
+                right=dict(heads=max(1, sz["width"] // 256), dim=128, vdim=256, gate_cap=15.0))
+    mlp = dict(kind="dense", ff=sz["ff"])
+    layers = [dict(type="parallel", mixer=pair, mlp=mlp), dict(type="attention", mixer=attention, mlp=mlp)] * (DESIGN_LAYERS // 2)
+    butolorn = dict(architecture="Butolorn", vocab=DESIGN_VOCAB, width=sz["width"], norm=dict(eps=1e-6),
+                    embedding=dict(scale=1.0), token_side=dict(dim=64), layers=layers, loop=dict(start=0, stop=0, times=1))
+    return penasun, config_from_dict(butolorn)
+
+
 def compare_designs(args) -> int:
     import torch
     import hector_engine_amd as he
@@ -217,16 +237,17 @@ def compare_designs(args) -> int:
         return out
 
     result = {}
+    beside = "penasun" if args.design == "butolorn" else "qwen2"
     chosen = [n for n in DESIGN_SIZES if not args.design_sizes or n in args.design_sizes.split(",")]
     for name in chosen:
         sz = DESIGN_SIZES[name]
         result[name] = {"sizes": sz}
-        configs = design_configs(sz) if args.design == "volonex" else penasun_configs(sz)
-        for design, config in zip(("qwen2", args.design), configs):
+        configs = {"volonex": design_configs, "penasun": penasun_configs, "butolorn": butolorn_configs}[args.design](sz)
+        for design, config in zip((beside, args.design), configs):
             progress(f"{name} {design}")
             result[name][design] = measure(config, False)
             result[name][design].update(measure(config, True))
-    print(json.dumps({"metric": "design_comparison", "design": args.design, "beside": "qwen2", "dtype": "bf16",
+    print(json.dumps({"metric": "design_comparison", "design": args.design, "beside": beside, "dtype": "bf16",
                       "data": "synthetic", "layers": DESIGN_LAYERS, "vocab": DESIGN_VOCAB, "prompt": prompt_len,
                       "batch": batch, "steps": steps, "sizes": result}))
     return 0
@@ -262,8 +283,8 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     ap.add_argument("--design-sizes", default="", help=f"with --design: only these of {', '.join(DESIGN_SIZES)}")
-    ap.add_argument("--design", choices=["volonex", "penasun"], default=None,
-                    help="instead of the run above: this design beside Qwen2 at equal layer sizes, prompt and "
+    ap.add_argument("--design", choices=["volonex", "penasun", "butolorn"], default=None,
+                    help="instead of the run above: this design beside Qwen2 (butolorn: beside Penasun) at equal layer sizes, prompt and "
                          "one-token steps, throughput and mean time per kind of kernel")
     args = ap.parse_args()
     if args.design:
