@@ -56,6 +56,10 @@ int he_add_dyt(void* resid_f32, const void* delta, float delta_scale, const void
 int he_rmsnorm_rows(void* out, const void* x, const void* weight, int rows, int D,
                     int64_t x_stride, int64_t out_stride, float eps, int dtype, int w_dtype,
                     void* stream);
+// x[r, 0:D1] and x[r, col2:col2+D2] of rows `stride` elements apart, each divided by its own root mean square
+// (eps inside the root) and multiplied by its gain (w1, w2; null: 1), in place, one launch.
+int he_rmsnorm_row_pair(void* x, const void* w1, int D1, const void* w2, int D2, int col2, int rows, int64_t stride,
+                        float eps, int dtype, int w_dtype, void* stream);
 
 // ---- matrix products: C[M,N] = A[M,K] * W[N,K]^T (+ bias) -------------------
 // he_gemm_plain: fp32 FMA sums in one fixed order per element (segments of 128 k, each a chain in
@@ -236,7 +240,8 @@ int he_gated_group_norm(void* out, const void* y_f32, const void* z, int64_t z_s
 // he_mlstm_gates: out_f32 [rows, 2 H] = the logarithms of the input gates (cap tanh((x + b) / cap)) and of the forget
 // gates (logsigmoid of the same bounded number) from their fp32 pre-activations x [rows, 2 H]; cap <= 0: unbounded.
 // he_mlstm_scan: y_f32 [rows, H dv] from q, k [rows, H dk] and v [rows, H dv] (views of rows in_stride elements
-// apart) and the gates' logarithms; S, n and m of a sequence live at state_offset of its row of `state`,
+// apart) and the gates' logarithms (raw_gates: their pre-activations, with gate_bias and cap as he_mlstm_gates takes
+// them, and the logarithms are formed inside); S, n and m of a sequence live at state_offset of its row of `state`,
 // he_mlstm_state_floats(H, dk, dv) floats, zeros at a sequence's start. dk up to 512.
 int64_t he_mlstm_state_floats(int H, int dk, int dv);
 int he_mlstm_gates(void* out_f32, const void* x_f32, const void* bias, int bias_dtype, int rows, int H, float cap,
@@ -244,7 +249,7 @@ int he_mlstm_gates(void* out_f32, const void* x_f32, const void* bias, int bias_
 int he_mlstm_scan(void* y_f32, const void* q, const void* k, const void* v, int64_t in_stride, const void* gates_f32,
                   void* state, int64_t state_stride, int64_t state_offset, const void* cu_seqlens,
                   const void* seq_slot, int rows, int num_seqs, int H, int dk, int dv, float q_scale, int dtype,
-                  void* stream);
+                  int raw_gates, const void* gate_bias, int bias_dtype, float cap, void* stream);
 
 // ---- routing and head combination (routing.hip) ---------------------------------
 // logits_f32 [rows][E], or null and x [rows][D] (x_dtype) with router_f32 [E][D]: the kernel forms the logits itself.

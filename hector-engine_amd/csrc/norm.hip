@@ -255,6 +255,45 @@ extern "C" int he_rmsnorm_rows(void* out, const void* x, const void* weight, int
   return he_check_launch("he_rmsnorm_rows");
 }
 
+// Two stretches of the same rows, each by a root mean square and a gain of its own, in place and in one launch:
+// columns [0, D1) with w1 and columns [col2, col2 + D2) with w2 (q and k as they lie behind one product).
+template <typename T>
+__global__ void rmsnorm_row_pair_kernel(T* __restrict__ x, const void* __restrict__ w1, int D1,
+                                        const void* __restrict__ w2, int D2, int col2, int w_dtype,
+                                        int64_t stride, float eps) {
+  __shared__ float scratch[16];
+  const bool second = blockIdx.y == 1;
+  const int D = second ? D2 : D1;
+  const void* w = second ? w2 : w1;
+  T* xi = x + blockIdx.x * stride + (second ? col2 : 0);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = to_float(xi[i]);
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / (float)D + eps);
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float g = w ? load_param(w, i, w_dtype) : 1.f;
+    xi[i] = from_float<T>(to_float(xi[i]) * inv * g);
+  }
+}
+
+extern "C" int he_rmsnorm_row_pair(void* x, const void* w1, int D1, const void* w2, int D2, int col2, int rows,
+                                   int64_t stride, float eps, int dtype, int w_dtype, void* stream) {
+  HE_REQUIRE(rows >= 0 && D1 > 0 && D2 > 0 && col2 >= D1 && stride >= (int64_t)col2 + D2,
+             "he_rmsnorm_row_pair: bad sizes rows=%d D1=%d D2=%d col2=%d", rows, D1, D2, col2);
+  HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_rmsnorm_row_pair: unknown dtype %d", dtype);
+  if (rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = norm_threads(D1 > D2 ? D1 : D2);
+  if (dtype == HE_BF16)
+    rmsnorm_row_pair_kernel<bf16_t><<<dim3(rows, 2), threads, 0, s>>>((bf16_t*)x, w1, D1, w2, D2, col2, w_dtype, stride, eps);
+  else
+    rmsnorm_row_pair_kernel<float><<<dim3(rows, 2), threads, 0, s>>>((float*)x, w1, D1, w2, D2, col2, w_dtype, stride, eps);
+  return he_check_launch("he_rmsnorm_row_pair");
+}
+
 // Rows x = r * gain whose scale is still owed: out = x / sqrt(sum(partials of the row) / D + eps).
 // The partial sums of squares (one per workgroup of the product that made the rows) are
 // added as that product's consumers add them: lanes over strided partials, then the wavefront.

@@ -63,10 +63,11 @@ _SIGNATURES = {
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_gated_group_norm": [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_int, c_int, c_int, c_int, c_f32, c_int, c_f32,
                             c_int, c_ptr],
+    "he_rmsnorm_row_pair": [c_ptr, c_ptr, c_int, c_ptr, c_int, c_int, c_int, c_i64, c_f32, c_int, c_int, c_ptr],
     "he_mlstm_state_floats": [c_int, c_int, c_int],
     "he_mlstm_gates": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_ptr],
     "he_mlstm_scan": [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_i64, c_i64, c_ptr, c_ptr, c_int, c_int,
-                      c_int, c_int, c_int, c_f32, c_int, c_ptr],
+                      c_int, c_int, c_int, c_f32, c_int, c_int, c_ptr, c_int, c_f32, c_ptr],
     "he_add_normed": [c_ptr, c_ptr, c_int, c_ptr, c_f32, c_ptr, c_f32, c_int, c_ptr, c_int, c_int, c_int, c_ptr],
     "he_unary_act": [c_ptr, c_ptr, c_i64, c_int, c_int, c_ptr],
     "he_token_gate": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],

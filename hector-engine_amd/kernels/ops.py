@@ -208,6 +208,21 @@ def rmsnorm_rows(out, x, weight, rows: int, D: int, x_stride: int, out_stride: i
                                  dtype_code(weight.dtype) if weight is not None else F32, _stream()))
 
 
+@_op("rmsnorm_row_pair")
+def rmsnorm_row_pair(x, w1, D1: int, w2, D2: int, col2: int, rows: int, eps: float) -> None:
+    """x[r, :D1] and x[r, col2:col2 + D2], each by its own root mean square and gain (w1, w2), in place, in one
+    launch. x: [rows, wide] with wide >= col2 + D2 (q and k as they lie behind one product)."""
+    if not x.is_cuda:
+        raise ValueError("x: expected a GPU tensor")
+    if x.dim() != 2 or x.stride(1) != 1 or x.shape[0] < rows or x.shape[1] < col2 + D2 or col2 < D1:
+        raise ValueError("rmsnorm_row_pair: the stretches do not lie in the rows")
+    _need(w1, "w1", shape=(D1,))
+    _need(w2, "w2", w1.dtype, (D2,))
+    L = _lib.load()
+    _lib.check(L.he_rmsnorm_row_pair(x.data_ptr(), w1.data_ptr(), D1, w2.data_ptr(), D2, col2, rows, x.stride(0),
+                                     float(eps), dtype_code(x.dtype), dtype_code(w1.dtype), _stream()))
+
+
 def gemm_plain_workspace_floats(M: int, N: int, K: int) -> int:
     """Floats of workspace with which gemm_plain runs a product of few rows through the kernels made
     for it (0: none needed)."""
@@ -742,10 +757,12 @@ def mlstm_gates(out, x, bias, rows: int, H: int, cap: float) -> None:
 
 @_op("mlstm_scan")
 def mlstm_scan(y, q, k, v, gates, state, state_offset: int, cu_seqlens, seq_slot, rows: int, num_seqs: int,
-               H: int, dk: int, dv: int, q_scale: float) -> None:
+               H: int, dk: int, dv: int, q_scale: float, raw_gates: bool = False, gate_bias=None, cap: float = 0.0) -> None:
     """y (fp32 [rows, H dv]) = the matrix memory's answers to q, after each row's k and v went in under the
     row's gates (gates: fp32 [rows, 2 H], the logarithms). q, k [rows, H dk] and v [rows, H dv] are views of
-    the same wider rows; the memory lives at byte state_offset of a sequence's row of `state` and is carried on."""
+    the same wider rows; the memory lives at byte state_offset of a sequence's row of `state` and is carried on.
+    raw_gates: `gates` holds the pre-activations, and the kernel forms the logarithms itself from them, gate_bias
+    ([2 H] or None) and cap, with mlstm_gates' arithmetic."""
     _need(y, "y", torch.float32, (None, H * dv))
     _need(gates, "gates", torch.float32, (None, 2 * H))
     stride = q.stride(0)
@@ -762,11 +779,14 @@ def mlstm_scan(y, q, k, v, gates, state, state_offset: int, cu_seqlens, seq_slot
     _need(seq_slot, "seq_slot", torch.int32)
     if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs:
         raise ValueError("mlstm_scan: metadata shorter than the step")
+    if gate_bias is not None:
+        _need(gate_bias, "gate_bias", None, (2 * H,))
     L = _lib.load()
     _lib.check(L.he_mlstm_scan(y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, gates.data_ptr(),
                                state.data_ptr(), state.stride(0), state_offset, cu_seqlens.data_ptr(),
                                seq_slot.data_ptr(), rows, num_seqs, H, dk, dv, float(q_scale), dtype_code(q.dtype),
-                               _stream()))
+                               int(raw_gates), _ptr(gate_bias), dtype_code(gate_bias.dtype) if gate_bias is not None else F32,
+                               float(cap), _stream()))
 
 
 @_op("route_tokens")

@@ -320,10 +320,10 @@ class Attention(Mixer):
         if self.qk_norm:
             # each token's q (all heads at once), and its k, by a root mean square of their own, in place
             wide = qkv.stride(0)
-            ops.rmsnorm_rows(qkv, qkv, self.q_norm_w, rows, H * hd, wide, wide, self.qk_norm_eps)
             if writes:
-                kq = qkv.reshape(-1)[H * hd:]       # the same rows, begun at their k columns
-                ops.rmsnorm_rows(kq, kq, self.k_norm_w, rows, KVH * hd, wide, wide, self.qk_norm_eps)
+                ops.rmsnorm_row_pair(qkv, self.q_norm_w, H * hd, self.k_norm_w, KVH * hd, H * hd, rows, self.qk_norm_eps)
+            else:
+                ops.rmsnorm_rows(qkv, qkv, self.q_norm_w, rows, H * hd, wide, wide, self.qk_norm_eps)
         if not fused_bias:
             q_cols, kv_cols = H * hd, KVH * hd
             qv = qkv[:, :q_cols].unflatten(1, (H, hd))

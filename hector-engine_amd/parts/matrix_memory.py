@@ -10,9 +10,9 @@ With H heads, keys of dk and values of dv dims (all from n, the mixer's input):
     out = W_o (rms over each head of y * norm * sigmoid(g))
 S, n and m start at zero and live in 32-bit floats in the sequence's row of the cache's state area,
 which the kernel addresses on the device through the step's slots: prompt steps, one-token steps, mixed
-steps and replayed graphs run the same launches. The two gates' weights are kept in 32 bits and their
-product is a 32-bit product also under bfloat16 activations: what enters the recurrence's exponentials
-is never rounded to 16 bits.
+steps and replayed graphs run the same launches. The two gates' product has 32-bit sums and a 32-bit
+result also under bfloat16 activations and weights: what enters the recurrence's exponentials is never
+rounded to 16 bits.
 
 names: the suffixes of its tensors (q, k, v, g, o, norm, i, f, i_bias, f_bias)."""
 from __future__ import annotations
@@ -82,7 +82,9 @@ class MatrixMemory(Mixer):
         self.qkvg = Linear(torch.cat(ws, 0).contiguous())
         del ws
         f32 = torch.float32
-        self.gates = Linear(torch.cat([tensors[n["i"]].to(f32), tensors[n["f"]].to(f32)], 0).contiguous())
+        # the gates' rows stay in the stored dtype: products of bfloat16 numbers are exact in 32 bits, and the sums
+        # and the result are 32-bit (out_dtype below), so nothing that enters the exponentials is rounded to 16 bits
+        self.gates = Linear(torch.cat([tensors[n["i"]], tensors[n["f"]]], 0).contiguous())
         self.gate_bias = torch.cat([tensors[n["i_bias"]].to(f32), tensors[n["f_bias"]].to(f32)], 0).contiguous()
         self.o_proj = Linear(tensors[n["o"]])
         self.norm = tensors[n["norm"]]
@@ -94,13 +96,13 @@ class MatrixMemory(Mixer):
         if ops.mlstm_state_floats(H, dk, dv) != self._state_floats():
             raise RuntimeError(f"{self.prefix}: the kernel's state layout differs from the cache's")
         proj = self.qkvg(x, rows, ctx)                                   # [rows, q | k | v | g]
-        pre = self.gates(x, rows, ctx, out_dtype=torch.float32)          # [rows, i | f], 32-bit
-        ops.mlstm_gates(pre, pre, self.gate_bias, rows, H, self.cap)
+        pre = self.gates(x, rows, ctx, out_dtype=torch.float32)          # [rows, i | f], 32-bit; the scan bounds them
         y = ctx.alloc((rows, H * dv), torch.float32)
         if ctx.padded:
             y.zero_()           # the scan writes the rows of sequences only
         ops.mlstm_scan(y, proj[:, :H * dk], proj[:, H * dk:2 * H * dk], proj[:, 2 * H * dk:2 * H * dk + H * dv], pre,
-                       cache.state, 0, ctx.cu_seqlens, ctx.seq_slot, rows, ctx.num_seqs, H, dk, dv, self.q_scale)
+                       cache.state, 0, ctx.cu_seqlens, ctx.seq_slot, rows, ctx.num_seqs, H, dk, dv, self.q_scale,
+                       raw_gates=True, gate_bias=self.gate_bias, cap=self.cap)
         g = ctx.alloc((rows, H * dv))
         ops.gated_group_norm(g, y, proj[:, 2 * H * dk + H * dv:], self.norm, rows, H, self.eps, gate_after=True,
                              out_scale=self.out_scale * out_scale)

@@ -255,6 +255,29 @@ def test_a_norm_over_the_whole_projection_inside_wider_rows(ops, dtype):
     assert torch.allclose(got[:, :Q], P.rms(x[:, :Q].double(), 1e-5) * wq.double(), rtol=tol, atol=tol)
     assert torch.allclose(got[:, Q:Q + K], P.rms(x[:, Q:Q + K].double(), 1e-5) * wk.double(), rtol=tol, atol=tol)
     assert torch.equal(got[:, Q + K:], x[:, Q + K:].double())                    # the rest of the rows stays
+    both = dev(x.clone())
+    ops.rmsnorm_row_pair(both, dev(wq), Q, dev(wk), K, Q, rows, 1e-5)            # the two in one launch: the same bits
+    assert torch.equal(both, d)
+
+
+def test_the_scan_forms_the_gates_logarithms_itself(ops):
+    """Given the pre-activations, the bias and the bound, the scan gives the bits it gives from logarithms made beforehand."""
+    H, dk, dv, rows = 3, 16, 24, 75
+    x = dev(rnd(rows, 2 * H * dk + H * dv, seed=1).to(torch.bfloat16))
+    pre, bias = dev(rnd(rows, 2 * H, seed=2, scale=4.0)), dev(rnd(2 * H, seed=3))
+    cu, slot = i32([0, 40, rows]), i32([1, 0])
+    outs = []
+    for raw in (False, True):
+        state = torch.zeros(2, 4 * ops.mlstm_state_floats(H, dk, dv), dtype=torch.uint8, device="cuda")
+        gates = pre
+        if not raw:
+            gates = torch.empty_like(pre)
+            ops.mlstm_gates(gates, pre, bias, rows, H, 7.0)
+        y = torch.empty(rows, H * dv, device="cuda")
+        ops.mlstm_scan(y, x[:, :H * dk], x[:, H * dk:2 * H * dk], x[:, 2 * H * dk:], gates, state, 0, cu, slot, rows, 2, H, dk, dv,
+                       0.25, raw_gates=raw, gate_bias=bias if raw else None, cap=7.0 if raw else 0.0)
+        outs.append((y, state))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
 
 
 # ------------------------------------------------------------------ whole models
