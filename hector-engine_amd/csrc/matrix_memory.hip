@@ -354,6 +354,104 @@ __global__ void __launch_bounds__(256) mlstm_scan_kernel(float* __restrict__ y, 
   }
 }
 
+template <typename T>
+__device__ __forceinline__ void mm_load8(float* dst, const T* p, int have, bool vec) {
+  if (vec && sizeof(T) == 2) {
+    mm_unpack<T>(dst, *reinterpret_cast<const mm_piece*>(p));
+  } else if (vec) {
+    mm_unpack<T>(dst, *reinterpret_cast<const mm_piece*>(p));
+    mm_unpack<T>(dst + 4, *reinterpret_cast<const mm_piece*>((const float*)p + 4));
+  } else {
+#pragma unroll
+    for (int e = 0; e < MM_NPT; ++e) dst[e] = e < have ? to_float(p[e]) : 0.f;
+  }
+}
+
+// Steps that bring every sequence one row: the same workgroups and threads, without the staging. A thread reads its
+// own key dims of q and k, its value and the head's gates straight from memory and forms the row's exponentials
+// itself; every product and sum is the one the kernel above forms, in the same order, so a row's result has the
+// same bits whichever of the two ran it.
+template <typename T>
+__global__ void __launch_bounds__(256) mlstm_step_kernel(float* __restrict__ y, const T* __restrict__ q, const T* __restrict__ k,
+                                                         const T* __restrict__ v, int64_t in_stride,
+                                                         const float* __restrict__ gates, uint8_t* __restrict__ state,
+                                                         int64_t state_stride, int64_t state_offset,
+                                                         const int32_t* __restrict__ cu_seqlens,
+                                                         const int32_t* __restrict__ seq_slot, int H, int dk, int dv, int NG,
+                                                         int PB, float q_scale, int vec, int raw_gates,
+                                                         const void* __restrict__ gate_bias, int bias_dtype, float cap) {
+  const int seq = blockIdx.z, h = blockIdx.y;
+  const int slot = seq_slot[seq];
+  const int r0 = cu_seqlens[seq], r1 = cu_seqlens[seq + 1];
+  if (slot < 0 || r0 >= r1) return;
+  const int c = threadIdx.x / NG, j = threadIdx.x % NG;
+  const int col = blockIdx.x * PB + c;
+  const bool active = c < PB && col < dv;
+  const int colc = active ? col : 0;
+  const int dkp = NG * MM_NPT;
+  const int d0 = j * MM_NPT;
+  const int have = dk - d0 < 0 ? 0 : (dk - d0 > MM_NPT ? MM_NPT : dk - d0);
+  const bool full = vec && have == MM_NPT;
+  const int dlo = have > 0 ? d0 : 0;     // a thread without key dims reads the row's first ones and drops them
+  float* st = reinterpret_cast<float*>(state + (int64_t)slot * state_stride + state_offset);
+  float* sp = st + ((int64_t)h * dv + colc) * dkp + d0;
+  float* aux = st + (int64_t)H * dv * dkp + ((int64_t)h * gridDim.x + blockIdx.x) * (dkp + 4);
+  float* np = aux + d0;
+  float* mp = aux + dkp;
+  float S[MM_NPT], nn[MM_NPT];
+  {
+    const float4 a = *reinterpret_cast<const float4*>(sp), b = *reinterpret_cast<const float4*>(sp + 4);
+    S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = b.x; S[5] = b.y; S[6] = b.z; S[7] = b.w;
+    const float4 e = *reinterpret_cast<const float4*>(np), f = *reinterpret_cast<const float4*>(np + 4);
+    nn[0] = e.x; nn[1] = e.y; nn[2] = e.z; nn[3] = e.w; nn[4] = f.x; nn[5] = f.y; nn[6] = f.z; nn[7] = f.w;
+  }
+  float m = *mp;
+  for (int r = r0; r < r1; ++r) {
+    float qc[MM_NPT], kc[MM_NPT];
+    const int64_t at = (int64_t)r * in_stride;
+    mm_load8(qc, q + at + (int64_t)h * dk + dlo, have, full);
+    mm_load8(kc, k + at + (int64_t)h * dk + dlo, have, full);
+#pragma unroll
+    for (int e = 0; e < MM_NPT; ++e) {
+      qc[e] = have > 0 ? qc[e] * q_scale : 0.f;
+      kc[e] = have > 0 ? kc[e] : 0.f;
+    }
+    const float vc = to_float(v[at + (int64_t)h * dv + colc]);
+    float ig = gates[(int64_t)r * 2 * H + h], fg = gates[(int64_t)r * 2 * H + H + h];
+    if (raw_gates) {
+      ig = mm_gate_log(ig + (gate_bias ? load_param(gate_bias, h, bias_dtype) : 0.f), cap, false);
+      fg = mm_gate_log(fg + (gate_bias ? load_param(gate_bias, H + h, bias_dtype) : 0.f), cap, true);
+    }
+    const float mn = fmaxf(fg + m, ig);
+    const float a = expf(fg + m - mn), b = expf(ig - mn);
+    m = mn;
+    float y0 = 0.f, y1 = 0.f, n0 = 0.f, n1 = 0.f;
+#pragma unroll
+    for (int e = 0; e < MM_NPT; e += 2) {
+      const float bk0 = b * kc[e], bk1 = b * kc[e + 1];
+      S[e] = fmaf(a, S[e], bk0 * vc);
+      S[e + 1] = fmaf(a, S[e + 1], bk1 * vc);
+      nn[e] = fmaf(a, nn[e], bk0);
+      nn[e + 1] = fmaf(a, nn[e + 1], bk1);
+      y0 = fmaf(S[e], qc[e], y0);
+      y1 = fmaf(S[e + 1], qc[e + 1], y1);
+      n0 = fmaf(nn[e], qc[e], n0);
+      n1 = fmaf(nn[e + 1], qc[e + 1], n1);
+    }
+    const float py = mm_group_sum(y0 + y1, NG), pn = mm_group_sum(n0 + n1, NG);
+    if (active && j == 0) y[(int64_t)r * H * dv + (int64_t)h * dv + col] = py / (fmaxf(fabsf(pn), expf(-m)) + 1e-6f);
+  }
+  if (active) {
+    *reinterpret_cast<float4*>(sp) = make_float4(S[0], S[1], S[2], S[3]);
+    *reinterpret_cast<float4*>(sp + 4) = make_float4(S[4], S[5], S[6], S[7]);
+  }
+  if (c == 0) {
+    *reinterpret_cast<float4*>(np) = make_float4(nn[0], nn[1], nn[2], nn[3]);
+    *reinterpret_cast<float4*>(np + 4) = make_float4(nn[4], nn[5], nn[6], nn[7]);
+    if (j == 0) *mp = m;
+  }
+}
+
 extern "C" int he_mlstm_scan(void* y_f32, const void* q, const void* k, const void* v, int64_t in_stride,
                              const void* gates_f32, void* state, int64_t state_stride, int64_t state_offset,
                              const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs, int H, int dk, int dv,
@@ -372,14 +470,24 @@ extern "C" int he_mlstm_scan(void* y_f32, const void* q, const void* k, const vo
   // whole 16-byte pieces of a row's q and k: every row and head starts aligned
   const int ve = 16 / esz;
   const bool vec = dk % ve == 0 && in_stride < (1 << 24) && (in_stride * esz) % 16 == 0 && (((uintptr_t)q | (uintptr_t)k) & 15) == 0;
+  const dim3 grid((dv + PB - 1) / PB, H, num_seqs);
+  hipStream_t s = (hipStream_t)stream;
+  if (rows <= num_seqs) {       // no sequence brings more than a row, or the few that do are walked row by row
+#define MM_STEP(T)                                                                                                       \
+  mlstm_step_kernel<T><<<grid, threads, 0, s>>>((float*)y_f32, (const T*)q, (const T*)k, (const T*)v, in_stride,          \
+                                                (const float*)gates_f32, (uint8_t*)state, state_stride, state_offset,    \
+                                                (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, H, dk, dv, NG, PB,  \
+                                                q_scale, (int)vec, raw_gates, gate_bias, bias_dtype, cap)
+    if (dtype == HE_BF16) MM_STEP(bf16_t); else MM_STEP(float);
+#undef MM_STEP
+    return he_check_launch("he_mlstm_scan");
+  }
   int TB = vec ? mm_block_rows(dk, dv, threads, 2 * dk / ve) : 0;
   const bool ahead = TB > 0;
   if (!ahead) TB = mm_block_rows(dk, dv, threads, 0);
   if (rows < TB) TB = rows;        // a step of few rows stages no more than it has
   const size_t lds = sizeof(float) * ((size_t)2 * TB * NG * MM_NPT + (size_t)2 * TB * PB + 6 * TB + 4);
   HE_REQUIRE(TB >= 1 && lds <= 64 * 1024, "he_mlstm_scan: a block of %d rows needs %zu bytes of LDS", TB, lds);
-  const dim3 grid((dv + PB - 1) / PB, H, num_seqs);
-  hipStream_t s = (hipStream_t)stream;
 #define MM_LAUNCH(T, AHEAD)                                                                                              \
   mlstm_scan_kernel<T, AHEAD><<<grid, threads, lds, s>>>((float*)y_f32, (const T*)q, (const T*)k, (const T*)v, in_stride, \
                                                          (const float*)gates_f32, (uint8_t*)state, state_stride,         \
