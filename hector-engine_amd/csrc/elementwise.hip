@@ -255,15 +255,53 @@ __global__ void unary_act_kernel(T* out, const T* x, int64_t n, int kind) {
   for (; i < n; i += stride) out[i] = from_float<T>(he_unary(to_float(x[i]), kind));
 }
 
+// The same over whole 16-byte pieces (8 bf16 or 4 fp32 a lane and turn); the launcher gives the rest to the kernel above.
+template <typename T>
+__global__ void unary_act_pieces_kernel(T* out, const T* x, int64_t pieces, int kind) {
+  constexpr int VE = 16 / sizeof(T);
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < pieces; i += stride) {
+    const uint4 v = reinterpret_cast<const uint4*>(x)[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (VE == 8) {
+        const float lo = he_unary(__uint_as_float(w[u] << 16), kind), hi = he_unary(__uint_as_float(w[u] & 0xffff0000u), kind);
+        o[u] = (uint32_t)float_to_bf16_bits(lo) | ((uint32_t)float_to_bf16_bits(hi) << 16);
+      } else {
+        o[u] = __float_as_uint(he_unary(__uint_as_float(w[u]), kind));
+      }
+    }
+    reinterpret_cast<uint4*>(out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 extern "C" int he_unary_act(void* out, const void* x, int64_t n, int kind, int dtype, void* stream) {
   HE_REQUIRE(n >= 0 && kind >= 0 && kind <= 3, "he_unary_act: bad size or kind %d", kind);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_unary_act: unknown dtype %d", dtype);
   if (n == 0) return 0;
-  int64_t blocks = (n + 255) / 256;
-  if (blocks > 65535) blocks = 65535;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == HE_BF16) unary_act_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, n, kind);
-  else unary_act_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)x, n, kind);
+  const int ve = dtype == HE_BF16 ? 8 : 4;
+  int64_t done = 0;
+  if ((((uintptr_t)out | (uintptr_t)x) & 15) == 0 && n >= ve) {
+    const int64_t pieces = n / ve;
+    int64_t blocks = (pieces + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    if (dtype == HE_BF16) unary_act_pieces_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)out, (const bf16_t*)x, pieces, kind);
+    else unary_act_pieces_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)out, (const float*)x, pieces, kind);
+    done = pieces * ve;
+    if (done == n) return he_check_launch("he_unary_act");
+  }
+  const int64_t rest = n - done;
+  int64_t blocks = (rest + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  const int esz = dtype == HE_BF16 ? 2 : 4;
+  void* o = (char*)out + done * esz;
+  const void* xi = (const char*)x + done * esz;
+  if (dtype == HE_BF16) unary_act_kernel<bf16_t><<<(int)blocks, 256, 0, s>>>((bf16_t*)o, (const bf16_t*)xi, rest, kind);
+  else unary_act_kernel<float><<<(int)blocks, 256, 0, s>>>((float*)o, (const float*)xi, rest, kind);
   return he_check_launch("he_unary_act");
 }
 

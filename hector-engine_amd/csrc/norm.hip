@@ -458,6 +458,83 @@ __global__ void add_normed_kernel(float* __restrict__ resid, const TD* __restric
   }
 }
 
+// Four neighbouring elements at once (16 bytes of fp32, 8 of bf16)
+__device__ __forceinline__ void pn_load4(float* dst, const float* p) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+}
+__device__ __forceinline__ void pn_load4(float* dst, const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  dst[0] = __uint_as_float(v.x << 16); dst[1] = __uint_as_float(v.x & 0xffff0000u);
+  dst[2] = __uint_as_float(v.y << 16); dst[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+__device__ __forceinline__ void pn_store4(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void pn_store4(bf16_t* p, const float* v) {
+  uint2 o;
+  o.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+  o.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+  *reinterpret_cast<uint2*>(p) = o;
+}
+
+// The same for rows whose width is a multiple of 4 and whose buffers begin on 16 bytes: a thread holds runs of four
+// neighbouring elements, and every load and store moves a run (the kernel above moves 2 or 4 bytes a lane).
+template <typename TD, typename TO>
+__global__ void add_normed_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta, const void* __restrict__ post_w,
+                                      float post_eps, const void* __restrict__ next_w, float next_eps, int w_dtype,
+                                      TO* __restrict__ out, int D) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* r = resid + row * D;
+  const TD* d = delta ? delta + row * D : nullptr;
+  float x[PN_EPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PN_EPT / 4; ++e) {
+    const int i = (threadIdx.x + e * blockDim.x) * 4;
+    if (d && i < D) pn_load4(x + 4 * e, d + i);
+    else x[4 * e] = x[4 * e + 1] = x[4 * e + 2] = x[4 * e + 3] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ss = fmaf(x[4 * e + u], x[4 * e + u], ss);
+  }
+  float inv = 1.f;
+  if (d && post_w) inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)D + post_eps);
+  ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < PN_EPT / 4; ++e) {
+    const int i = (threadIdx.x + e * blockDim.x) * 4;
+    if (i < D) {
+      float old[4];
+      pn_load4(old, r + i);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float g = (d && post_w) ? load_param(post_w, i + u, w_dtype) : 1.f;
+        x[4 * e + u] = d ? old[u] + x[4 * e + u] * inv * g : old[u];
+      }
+      if (d) pn_store4(r + i, x + 4 * e);
+    } else {
+      x[4 * e] = x[4 * e + 1] = x[4 * e + 2] = x[4 * e + 3] = 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ss = fmaf(x[4 * e + u], x[4 * e + u], ss);
+  }
+  if (out == nullptr) return;
+  float inv2 = 1.f;
+  if (next_w) inv2 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)D + next_eps);
+  TO* o = out + row * D;
+#pragma unroll
+  for (int e = 0; e < PN_EPT / 4; ++e) {
+    const int i = (threadIdx.x + e * blockDim.x) * 4;
+    if (i < D) {
+      float y[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) y[u] = next_w ? x[4 * e + u] * inv2 * load_param(next_w, i + u, w_dtype) : x[4 * e + u];
+      pn_store4(o + i, y);
+    }
+  }
+}
+
 extern "C" int he_add_normed(void* resid_f32, const void* delta, int delta_dtype, const void* post_weight, float post_eps,
                              const void* next_weight, float next_eps, int w_dtype, void* out, int out_dtype, int rows,
                              int D, void* stream) {
@@ -476,6 +553,17 @@ extern "C" int he_add_normed(void* resid_f32, const void* delta, int delta_dtype
   add_normed_kernel<TD, TO><<<rows, threads, 0, s>>>((float*)resid_f32, (const TD*)delta, post_weight, post_eps, \
                                                      next_weight, next_eps, w_dtype, (TO*)out, D)
   const bool db = delta != nullptr && delta_dtype == HE_BF16, ob = out != nullptr && out_dtype == HE_BF16;
+  if (D % 4 == 0 && (((uintptr_t)resid_f32 | (uintptr_t)delta | (uintptr_t)out) & 15) == 0) {
+#define PN_VEC(TD, TO)                                                                                                \
+  add_normed_vec_kernel<TD, TO><<<rows, threads, 0, s>>>((float*)resid_f32, (const TD*)delta, post_weight, post_eps,   \
+                                                         next_weight, next_eps, w_dtype, (TO*)out, D)
+    if (db && ob) PN_VEC(bf16_t, bf16_t);
+    else if (db) PN_VEC(bf16_t, float);
+    else if (ob) PN_VEC(float, bf16_t);
+    else PN_VEC(float, float);
+#undef PN_VEC
+    return he_check_launch("he_add_normed");
+  }
   if (db && ob) PN_LAUNCH(bf16_t, bf16_t);
   else if (db) PN_LAUNCH(bf16_t, float);
   else if (ob) PN_LAUNCH(float, bf16_t);
