@@ -82,6 +82,8 @@ def _attention(data: dict, where: str) -> ButolornAttention:
     heads = read_field(data, "heads", int)
     dim = read_field(data, "dim", int)
     rot = read_object(data, "rot", None)
+    if rot is not None and read_field(rot, "dims", int, dim) == 0:
+        rot = None          # no dimension is rotated
     a = ButolornAttention(heads=heads, kv_heads=read_field(data, "kv_heads", int, heads), dim=dim,
                           vdim=read_field(data, "vdim", int, dim), scale=read_field(data, "scale", float),
                           rot_base=0.0 if rot is None else read_field(rot, "base", float),

@@ -83,6 +83,8 @@ def test_defaults_for_what_a_layer_leaves_out():
     assert cfg.layers[0].mixer.left_scale == 1.0 and cfg.side_dim == 0 and cfg.embedding_scale == 1.0
     spec = build_model(cfg, BuildEnv(torch.device("cpu"), torch.float32)).tensor_specs()
     assert "side.embed" not in spec and "l0.side.gate" not in spec
+    d["layers"][2]["mixer"]["left"]["rot"]["dims"] = 0                 # no dimension rotated: the same as no 'rot'
+    assert config_from_dict(d).layers[2].mixer.left.rot_dims == 0
 
 
 @pytest.mark.parametrize("path,value,word", [
