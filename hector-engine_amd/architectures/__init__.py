@@ -1,2 +1,2 @@
 """Architectures known to the registry."""
-from . import butolorn, penasun, qwen2, volonex  # noqa: F401
+from . import butolorn, domorax, penasun, qwen2, volonex  # noqa: F401

@@ -101,7 +101,8 @@ __device__ __forceinline__ void ap_fetch(float (&kv)[AP_GROUP][NPL], float (&vv)
 template <typename T, int NPL>
 __device__ __forceinline__ void ap_page(ApState<NPL>& st, const float (&qv)[NPL], const T* kpool,
                                         const T* vpool, int page, int num_pages, int KVH, int kvh, int hd,
-                                        int j_lo, int j_hi, float scale, int lane, int npl) {
+                                        int j_lo, int j_hi, float scale, int lane, int npl, float slope = 0.f,
+                                        int p = 0) {
   st.m = -INFINITY;
   st.l = 0.f;
 #pragma unroll
@@ -121,13 +122,15 @@ __device__ __forceinline__ void ap_page(ApState<NPL>& st, const float (&qv)[NPL]
     ap_fetch<T, NPL>(kb, vb, kpage, vpage, j0 + AP_GROUP, j_hi, KS, NT, lane, npl, hd);
     float sc[AP_GROUP];
 #pragma unroll
-    for (int g = 0; g < AP_GROUP; ++g) sc[g] = ap_score<NPL>(qv, ka[g], scale, lane, npl, hd);
+    for (int g = 0; g < AP_GROUP; ++g)
+      sc[g] = fmaf(slope, (float)(j0 + g - p), ap_score<NPL>(qv, ka[g], scale, lane, npl, hd));
 #pragma unroll
     for (int g = 0; g < AP_GROUP; ++g)
       if (j0 + g <= j_hi) ap_update<NPL>(st, sc[g], va[g], lane, npl, hd);
     ap_fetch<T, NPL>(ka, va, kpage, vpage, j0 + 2 * AP_GROUP, j_hi, KS, NT, lane, npl, hd);
 #pragma unroll
-    for (int g = 0; g < AP_GROUP; ++g) sc[g] = ap_score<NPL>(qv, kb[g], scale, lane, npl, hd);
+    for (int g = 0; g < AP_GROUP; ++g)
+      sc[g] = fmaf(slope, (float)(j0 + AP_GROUP + g - p), ap_score<NPL>(qv, kb[g], scale, lane, npl, hd));
 #pragma unroll
     for (int g = 0; g < AP_GROUP; ++g)
       if (j0 + AP_GROUP + g <= j_hi) ap_update<NPL>(st, sc[g], vb[g], lane, npl, hd);
@@ -153,6 +156,7 @@ struct ApExtras {
   int sinks_dtype;
   const void* gate;      // gate[row * gate_stride + h] in the activation dtype, or null
   int64_t gate_stride;
+  const float* slopes;   // [H] or null: the score of key j for the query at p loses slopes[h] * (p - j)
 };
 template <typename T, int NPL>
 __device__ __forceinline__ float ap_finish(ApState<NPL>& total, const ApExtras& ex, int64_t row, int h) {
@@ -198,6 +202,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   const int p = positions[row];
   const int slot = seq_slot[seq];
   const int kvh = h / (H / KVH);
+  const float slope = ex.slopes ? ex.slopes[h] : 0.f;
   const int first = ap_first(p, window, chunk);
   const int32_t* pt = page_table + (int64_t)slot * max_blocks;
   const int c_first = first >> HE_PAGE_SHIFT, c_last = p >> HE_PAGE_SHIFT;
@@ -214,7 +219,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   if (split) {
     const int c = c_first + blockIdx.z;
     ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
-               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl, slope, p);
     float* w = ws + ((row * H + h) * (int64_t)gridDim.z + blockIdx.z) * (hd + 2);
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(
   for (int i = 0; i < NPL; ++i) total.acc[i] = 0.f;
   for (int c = c_first; c <= c_last; ++c) {
     ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
-               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+               min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl, slope, p);
     ap_join(total, st);
   }
   const float gf = ap_finish<T, NPL>(total, ex, row, h);
@@ -262,6 +267,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
   const int npl = (hd + HE_WAVE - 1) / HE_WAVE;
   const int kvh = h / (H / KVH);
   const int n_rows = (int)min((int64_t)AP_ROWS, rows - row0);
+  const float slope = ex.slopes ? ex.slopes[h] : 0.f;
   const int seq0 = row_seq[row0], p0 = positions[row0];
   bool together = n_rows == AP_ROWS && seq0 >= 0;
   for (int r = 1; r < n_rows; ++r) together = together && row_seq[row0 + r] == seq0 && positions[row0 + r] == p0 + r;
@@ -300,7 +306,7 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
         load_q(qv, row);
         for (int c = first >> HE_PAGE_SHIFT; c <= (p >> HE_PAGE_SHIFT); ++c) {
           ap_page<T, NPL>(st, qv, kpool, vpool, pt[c], num_pages, KVH, kvh, hd, max(first, c << HE_PAGE_SHIFT),
-                          min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl);
+                          min(p, (c << HE_PAGE_SHIFT) + HE_PAGE_TOKENS - 1), scale, lane, npl, slope, p);
           ap_join(total, st);
         }
       }
@@ -347,7 +353,8 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
 #pragma unroll
         for (int g = 0; g < AP_GROUP; ++g)
 #pragma unroll
-          for (int r = 0; r < AP_ROWS; ++r) sc[g][r] = ap_score<NPL>(qv[r], ka[g], scale, lane, npl, hd);
+          for (int r = 0; r < AP_ROWS; ++r)
+            sc[g][r] = fmaf(slope, (float)(j0 + g - p0 - r), ap_score<NPL>(qv[r], ka[g], scale, lane, npl, hd));
 #pragma unroll
         for (int g = 0; g < AP_GROUP; ++g) {
           const int j = j0 + g;
@@ -359,7 +366,8 @@ __global__ __launch_bounds__(256) void attention_plain_rows_kernel(
 #pragma unroll
         for (int g = 0; g < AP_GROUP; ++g)
 #pragma unroll
-          for (int r = 0; r < AP_ROWS; ++r) sc[g][r] = ap_score<NPL>(qv[r], kb[g], scale, lane, npl, hd);
+          for (int r = 0; r < AP_ROWS; ++r)
+            sc[g][r] = fmaf(slope, (float)(j0 + AP_GROUP + g - p0 - r), ap_score<NPL>(qv[r], kb[g], scale, lane, npl, hd));
 #pragma unroll
         for (int g = 0; g < AP_GROUP; ++g) {
           const int j = j0 + AP_GROUP + g;
@@ -466,7 +474,7 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
                                   int H, int KVH, int hd, int window, int chunk, float scale,
                                   const void* sinks, int sinks_dtype, const void* gate,
                                   int64_t gate_stride, int dtype, int most_keys, void* workspace_f32,
-                                  int64_t workspace_floats, void* stream) {
+                                  int64_t workspace_floats, const void* slopes_f32, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0, "he_attention_plain: bad sizes");
   HE_REQUIRE(H % KVH == 0, "he_attention_plain: heads %d not a multiple of kv heads %d", H, KVH);
   HE_REQUIRE(hd <= AP_MAX_PER_LANE * HE_WAVE, "he_attention_plain: head_dim %d above %d", hd,
@@ -475,7 +483,7 @@ extern "C" int he_attention_plain(void* out, const void* q, const void* kpool, c
   HE_REQUIRE(sinks == nullptr || sinks_dtype == HE_BF16 || sinks_dtype == HE_F32,
              "he_attention_plain: unknown dtype %d of the sinks", sinks_dtype);
   if (rows == 0) return 0;
-  const ApExtras ex = {sinks, sinks_dtype, gate, gate_stride};
+  const ApExtras ex = {sinks, sinks_dtype, gate, gate_stride, (const float*)slopes_f32};
   // page by page in parallel when the caller brought room for it (the same bits either way)
   const int64_t need = he_attention_plain_workspace_floats(rows, H, hd, most_keys, window, chunk);
   const bool split = need > 0 && workspace_f32 != nullptr && workspace_floats >= need;

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 26
+#define HE_ABI_VERSION 27
 
 #ifdef __cplusplus
 extern "C" {
@@ -161,7 +161,9 @@ int he_attention_plain(void* out, const void* q, const void* kpool, const void* 
                        const void* page_table, int max_blocks, int num_pages, int rows, int H,
                        int KVH, int hd, int window, int chunk, float scale, const void* sinks,
                        int sinks_dtype, const void* gate, int64_t gate_stride, int dtype,
-                       int most_keys, void* workspace_f32, int64_t workspace_floats, void* stream);
+                       int most_keys, void* workspace_f32, int64_t workspace_floats, const void* slopes_f32,
+                       void* stream);
+// slopes_f32 (or null): one number a head; the score of key j for the query at p loses slope * (p - j).
 // bf16, one query row per sequence (decode): split over the keys, then merged. chunk, sinks and
 // gate (bf16 here) as he_attention_plain takes them; so does he_attention_prefill_bf16.
 int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const void* vpool,
@@ -222,7 +224,7 @@ int he_conv_state(void* out, const void* x, int64_t x_stride, const void* taps, 
                   int w_dtype, void* state, int64_t state_stride, const void* positions,
                   const void* row_seq, const void* seq_slot, const void* seq_start,
                   const void* cu_seqlens, int rows, int num_seqs, int C, int K, int all_single,
-                  int dtype, void* stream);
+                  int act, int dtype, void* stream);
 int64_t he_ssm_state_floats(int R, int P, int N);
 // xbc [rows][R P + 2 Q N]: x, then the Q groups' B vectors, then their C vectors; dt_in[row * dt_stride + r].
 // y [rows][R P] fp32 (rows without a sequence are not written). max_q_len: a bound on the rows a sequence brings (0: none).
@@ -256,7 +258,7 @@ int he_mlstm_scan(void* y_f32, const void* q, const void* k, const void* v, int6
 int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
                     const void* x, int x_dtype, const void* router_f32, int D,
                     const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
-                    int top, float scale, void* stream);
+                    int top, float scale, int normalize, void* stream);
 int he_routed_act(void* out, const void* gate_up, const void* dense_f32, const void* h, int rows, int real,
                   int I, int extra, int dtype, float alpha, float limit, float up_shift, void* stream);
 // For a step of very few rows (bf16): out[rows][D] = the weighted sum of the chosen experts' results alone, from
@@ -317,6 +319,47 @@ int he_token_gate(void* out, const void* x, const void* table, const void* ids, 
 int he_sigmoid_gate(void* x, const void* gate, int64_t gate_stride, int rows, int H, int hd, int vd, float scale,
                     int dtype, void* stream);
 int he_scaled_sum(void* out, const void* a, const void* b, int64_t n, float sa, float sb, int dtype, void* stream);
+
+// ---- a gated delta rule carried from token to token (delta_rule.hip) -------------------------------
+// y_f32 [rows, H e] from q, k [rows, G d] and v [rows, H e] (views of rows in_stride elements apart, head h reads the
+// q and k of group h / (H / G)), ba_f32 [rows, 2 H] (write strengths b, then decay inputs a) and per head a_log, dt_bias:
+// q, k to unit length (q times q_scale), beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)); S <- g S;
+// u = beta (v - S^T k); S <- S + k u^T; y = S^T q. S (fp32, he_delta_state_floats floats) lives at byte state_offset of the
+// sequence's row of the state area and is carried on.
+int64_t he_delta_state_floats(int H, int d, int e);
+int he_delta_scan(void* y_f32, const void* q, const void* k, const void* v, int64_t in_stride, const void* ba_f32,
+                  const void* a_log, const void* dt_bias, int w_dtype, void* state, int64_t state_stride,
+                  int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs, int H, int G,
+                  int d, int e, float q_scale, float unit_eps, int dtype, void* stream);
+
+// ---- norms over parts of a row (group_norm.hip) --------------------------------------------------------
+// resid += delta_scale * gn(delta) with gn the RMS norm in `groups` equal consecutive parts times weight (delta null:
+// nothing is added); then out (if given) = next_weight ? gn'(resid) : resid, in out_dtype.
+int he_add_group_normed(void* resid_f32, const void* delta, int delta_dtype, const void* weight, int w_dtype, int groups,
+                        float eps, float delta_scale, void* out, int out_dtype, const void* next_weight, int next_groups,
+                        float next_eps, int rows, int D, void* stream);
+// out = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e per row of W values; numbers = (a, b, c, e)
+int he_polynorm(void* out, const void* x, const void* numbers, int n_dtype, int rows, int W, float eps, int dtype,
+                void* stream);
+// rows [H q heads | G k heads] of d from `in` to rows [H q heads | G k heads | G v heads] of out (which may be in):
+// q and k heads RMS-normed with q_w / k_w [d]; copy_v: the k heads as they were become the v heads
+int he_qk_head_norm(void* out, int64_t out_stride, const void* in, int64_t in_stride, const void* q_w, const void* k_w, int w_dtype, int H, int G, int d,
+                    float eps, int copy_v, int rows, int dtype, void* stream);
+
+// ---- whole rows of the stream (stream_ops.hip) ---------------------------------------------------------
+// kept_f32 plane n - 1 = resid; resid = sum_{j < n} coeffs[j] * plane j
+int he_depth_mix(void* resid_f32, void* kept_f32, int64_t plane, const void* coeffs, int c_dtype, int n, int64_t count,
+                 void* stream);
+// out = a + sigmoid(x . g) * b, row by row
+int he_gated_add(void* out, const void* a, const void* b, const void* x, const void* g, int g_dtype, int rows, int D,
+                 int Dx, int dtype, void* stream);
+
+// ---- latent attention (latent.hip) ---------------------------------------------------------------------
+// out[r, h, n] = sum_k x[r, h, k] w[h][k][n]
+int he_head_product(void* out, int64_t o_row, int64_t o_head, const void* x, int64_t x_row, int64_t x_head, const void* w,
+                    int w_dtype, int rows, int H, int K, int N, int dtype, void* stream);
+int he_latent_pack(void* qkv, const void* q, const void* down, int64_t down_stride, int rows, int H, int d, int r,
+                   int rank, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

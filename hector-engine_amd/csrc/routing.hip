@@ -31,7 +31,8 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(
     float* __restrict__ dense, int32_t* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
     const void* __restrict__ x, int x_dtype, const float* __restrict__ router, int D,
-    const void* __restrict__ correction, int c_dtype, int E, int real, int groups, int keep, int top, float scale) {
+    const void* __restrict__ correction, int c_dtype, int E, int real, int groups, int keep, int top, float scale,
+    int normalize) {
   __shared__ float s_sh[ROUTE_MAX_EXPERTS];
   __shared__ float c_sh[ROUTE_MAX_EXPERTS];
   __shared__ float d_sh[ROUTE_MAX_EXPERTS + 1];
@@ -139,6 +140,7 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(
     }
     __syncthreads();
   }
+  float chosen_sum = 0.f;     // lane 0 of the first wavefront: the chosen outputs' scores, added in the order of the choice
   for (int k = 0; k < top; ++k) {
     float v = -INFINITY;
     int idx = 0x7fffffff;
@@ -161,6 +163,7 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(
       if (found) {
         c_sh[e] = NAN;
         d_sh[e < real ? e : real] += w;
+        chosen_sum += s_sh[e];
       }
       ids[row * top + k] = found ? e : -1;
       weights[row * top + k] = w;
@@ -168,14 +171,18 @@ __global__ __launch_bounds__(64 * ROUTE_WAVES) void route_kernel(
     __syncthreads();
   }
   if (lead) {
-    for (int e = lane; e <= real; e += 64) dense[row * (real + 1) + e] = d_sh[e];
+    // normalize: the chosen outputs' weights are made to sum to `scale` (the softmax over the chosen logits alone)
+    const float norm = normalize ? 1.f / __shfl(chosen_sum, 0) : 1.f;
+    for (int e = lane; e <= real; e += 64) dense[row * (real + 1) + e] = normalize ? d_sh[e] * norm : d_sh[e];
+    if (normalize)
+      for (int k = lane; k < top; k += 64) weights[row * top + k] *= norm;
   }
 }
 
 extern "C" int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32, const void* logits_f32,
                                const void* x, int x_dtype, const void* router_f32, int D,
                                const void* correction, int c_dtype, int rows, int E, int real, int groups, int keep,
-                               int top, float scale, void* stream) {
+                               int top, float scale, int normalize, void* stream) {
   HE_REQUIRE((logits_f32 != nullptr) != (x != nullptr), "he_route_tokens: give the logits, or the rows and the router");
   HE_REQUIRE(x == nullptr || (router_f32 != nullptr && D > 0 && (x_dtype == HE_BF16 || x_dtype == HE_F32)),
              "he_route_tokens: the router's matrix is missing");
@@ -188,7 +195,7 @@ extern "C" int he_route_tokens(void* dense_f32, void* ids_i32, void* weights_f32
   if (rows == 0) return 0;
   route_kernel<<<rows, 64 * ROUTE_WAVES, 0, (hipStream_t)stream>>>((float*)dense_f32, (int32_t*)ids_i32, (float*)weights_f32,
                                                      (const float*)logits_f32, x, x_dtype, (const float*)router_f32, D,
-                                                     correction, c_dtype, E, real, groups, keep, top, scale);
+                                                     correction, c_dtype, E, real, groups, keep, top, scale, normalize);
   return he_check_launch("he_route_tokens");
 }
 

@@ -11,7 +11,7 @@ __device__ __forceinline__ float ss_softplus(float z) { return z > 20.f ? z : lo
 
 // ---- causal convolution per channel ---------------------------------------------------------
 // out[row, c] = silu(bias[c] + sum_j taps[c, j] * u[pos - (K-1) + j, c]): the last tap weighs the
-// row's own input. Inputs before the step's first row of the sequence come from the carried inputs
+// row's own input (bias null: none; act 0: the sum as it is, without silu). Inputs before the step's first row of the sequence come from the carried inputs
 // (zeros at a sequence's start). SINGLE: every sequence brings one row, and the thread that computed
 // (row, c) also moves the carried inputs on; otherwise conv_carry_kernel does that afterwards.
 template <typename T, bool SINGLE>
@@ -20,7 +20,7 @@ __global__ void conv_taps_kernel(T* __restrict__ out, const T* __restrict__ x, i
                                  uint8_t* __restrict__ state, int64_t state_stride,
                                  const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
                                  const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_start,
-                                 int C, int K) {
+                                 int C, int K, int act) {
   const int64_t row = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -32,7 +32,7 @@ __global__ void conv_taps_kernel(T* __restrict__ out, const T* __restrict__ x, i
   }
   const int before = positions[row] - seq_start[seq];   // rows of the same sequence ahead of this one in the step
   float* hist = reinterpret_cast<float*>(state + (int64_t)slot * state_stride);
-  float acc = load_param(bias, c, w_dtype);
+  float acc = bias ? load_param(bias, c, w_dtype) : 0.f;
   for (int j = 0; j < K; ++j) {
     const int back = K - 1 - j;
     float u;
@@ -42,7 +42,7 @@ __global__ void conv_taps_kernel(T* __restrict__ out, const T* __restrict__ x, i
       u = hist[(int64_t)(K - 1 - (back - before)) * C + c];
     acc = fmaf(load_param(taps, (int64_t)c * K + j, w_dtype), u, acc);
   }
-  out[row * (int64_t)C + c] = from_float<T>(ss_silu(acc));
+  out[row * (int64_t)C + c] = from_float<T>(act ? ss_silu(acc) : acc);
   if (SINGLE) {
     for (int i = 0; i + 2 < K; ++i) hist[(int64_t)i * C + c] = hist[(int64_t)(i + 1) * C + c];
     if (K > 1) hist[(int64_t)(K - 2) * C + c] = to_float(x[row * x_stride + c]);
@@ -76,7 +76,7 @@ extern "C" int he_conv_state(void* out, const void* x, int64_t x_stride, const v
                              int w_dtype, void* state, int64_t state_stride, const void* positions,
                              const void* row_seq, const void* seq_slot, const void* seq_start,
                              const void* cu_seqlens, int rows, int num_seqs, int C, int K, int all_single,
-                             int dtype, void* stream) {
+                             int act, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && num_seqs >= 0 && C > 0 && K >= 1 && K <= 64, "he_conv_state: bad sizes rows=%d C=%d K=%d", rows,
              C, K);
   HE_REQUIRE(dtype == HE_BF16 || dtype == HE_F32, "he_conv_state: unknown dtype %d", dtype);
@@ -89,7 +89,7 @@ extern "C" int he_conv_state(void* out, const void* x, int64_t x_stride, const v
 #define CONV_LAUNCH(T, SINGLE)                                                                          \
   conv_taps_kernel<T, SINGLE><<<grid, threads, 0, s>>>(                                                 \
       (T*)out, (const T*)x, x_stride, taps, bias, w_dtype, (uint8_t*)state, state_stride,               \
-      (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)seq_start, C, K)
+      (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot, (const int32_t*)seq_start, C, K, act)
   if (dtype == HE_BF16) {
     if (all_single) CONV_LAUNCH(bf16_t, true); else CONV_LAUNCH(bf16_t, false);
   } else {
@@ -376,6 +376,7 @@ __global__ void gated_group_norm_kernel(T* __restrict__ out, const float* __rest
       v = v * ss_silu(g) * inv * load_param(weight, c0 + i, w_dtype);
     } else {
       v = v * inv * load_param(weight, c0 + i, w_dtype) * (out_scale / (1.f + expf(-g)));
+      if (gate_after == 2) v *= g;      // silu(g) = g * sigmoid(g)
     }
     out[row * W + c0 + i] = from_float<T>(v);
   }

@@ -7,7 +7,7 @@ import torch
 
 from ..cache.paged import RunPlan
 from ..kernels import ops
-from ..parts.base import BuildEnv, LayerCache, ModelSpec, ResidualStream, StepContext, build_part
+from ..parts.base import BuildEnv, LayerCache, ModelSpec, ResidualStream, StepContext, TensorSpec, build_part
 
 
 class DecoderModel:
@@ -19,6 +19,10 @@ class DecoderModel:
         self.final_norm = build_part("norm", spec.final_norm, spec.final_norm_prefix, env)
         self.head = build_part("head", spec.head, spec.head_prefix, env)
         self.schedule = list(spec.schedule)
+        self.depth_mix = list(spec.depth_mix) if spec.depth_mix else None
+        self.mix_coeffs: list[torch.Tensor] = []
+        if self.depth_mix is not None and len(self.depth_mix) != len(self.schedule):
+            raise ValueError(f"depth_mix names {len(self.depth_mix)} tensors for {len(self.schedule)} runs")
         for e, entry in enumerate(self.schedule):
             if not 0 <= entry.layer < len(self.blocks):
                 raise ValueError(f"schedule entry {e} names layer {entry.layer}, "
@@ -63,9 +67,13 @@ class DecoderModel:
         specs = {}
         for p in self.parts():
             specs.update(p.tensor_specs())
+        for e, name in enumerate(self.depth_mix or []):
+            # random models: mostly the newest result, a little of every earlier one
+            specs[name] = TensorSpec((e + 2,), ("gain", 1.0 / (e + 2), 0.25))
         return specs
 
     def bind(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.mix_coeffs = [tensors[name] for name in self.depth_mix or []]
         for p in self.parts():
             p.bind(tensors)
 
@@ -92,6 +100,11 @@ class DecoderModel:
             # the embedding's output, kept for the runs that start again from it
             embedded = ctx.alloc((rows, self.spec.hidden_size), torch.float32)
             embedded.copy_(resid)
+        kept = None
+        if self.depth_mix is not None:
+            # every run's result is kept for the step: plane 0 the embedding's output, plane e + 1 run e's
+            kept = ctx.alloc((len(self.schedule) + 1, rows, self.spec.hidden_size), torch.float32)
+            kept[0].copy_(resid)
         last = len(self.schedule) - 1
         for e, entry in enumerate(self.schedule):
             if entry.add_embedding:
@@ -104,8 +117,13 @@ class DecoderModel:
                     self.blocks[self.schedule[e + 1].layer].first_norm()
             else:
                 ctx.next_norm = self.final_norm if (ctx.want_all and n_want == rows) else None
+            if kept is not None:
+                ctx.next_norm = None            # the stream is mixed before anything reads it
             ctx.scratch.begin_layer()
             self.blocks[entry.layer].forward(stream, ctx, caches[e])
+            if kept is not None:
+                stream.prepared = stream.ready = None
+                ops.depth_mix(stream.materialize(ctx), kept, self.mix_coeffs[e], e + 2, rows)
         ctx.scratch.end_layers()
         ctx.next_norm = None
         if n_want == 0:

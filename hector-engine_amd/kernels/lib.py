@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 26
+EXPECTED_ABI = 27
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -57,7 +57,7 @@ _SIGNATURES = {
                           c_int, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_ptr, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_int, c_int, c_ptr],
     "he_conv_state": [c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_int, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr,
-                      c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
+                      c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_ssm_state_floats": [c_int, c_int, c_int],
     "he_ssm_scan": [c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_i64, c_i64, c_ptr, c_ptr,
                     c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
@@ -74,7 +74,18 @@ _SIGNATURES = {
     "he_sigmoid_gate": [c_ptr, c_ptr, c_i64, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr],
     "he_scaled_sum": [c_ptr, c_ptr, c_ptr, c_i64, c_f32, c_f32, c_int, c_ptr],
     "he_route_tokens": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_int, c_ptr, c_int, c_int, c_int, c_int,
-                        c_int, c_int, c_int, c_f32, c_ptr],
+                        c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_delta_state_floats": [c_int, c_int, c_int],
+    "he_delta_scan": [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_i64, c_i64, c_ptr, c_ptr,
+                      c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_int, c_ptr],
+    "he_add_group_normed": [c_ptr, c_ptr, c_int, c_ptr, c_int, c_int, c_f32, c_f32, c_ptr, c_int, c_ptr, c_int, c_f32,
+                            c_int, c_int, c_ptr],
+    "he_polynorm": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_int, c_ptr],
+    "he_qk_head_norm": [c_ptr, c_i64, c_ptr, c_i64, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_f32, c_int, c_int, c_int, c_ptr],
+    "he_depth_mix": [c_ptr, c_ptr, c_i64, c_ptr, c_int, c_int, c_i64, c_ptr],
+    "he_gated_add": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_head_product": [c_ptr, c_i64, c_i64, c_ptr, c_i64, c_i64, c_ptr, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
+    "he_latent_pack": [c_ptr, c_ptr, c_ptr, c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_ptr],
     "he_routed_act": [c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_f32, c_ptr],
     "he_chosen_experts": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_int,
                           c_int, c_f32, c_f32, c_f32, c_ptr],
@@ -82,7 +93,7 @@ _SIGNATURES = {
     "he_attention_plain_workspace_floats": [c_int, c_int, c_int, c_int, c_int, c_int],
     "he_attention_plain": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_ptr, c_int, c_ptr, c_i64,
-                           c_int, c_int, c_ptr, c_i64, c_ptr],
+                           c_int, c_int, c_ptr, c_i64, c_ptr, c_ptr],
     "he_attention_decode_bf16": [c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_ptr, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_int, c_ptr,
                                  c_i64, c_int, c_ptr, c_int, c_ptr, c_i64, c_ptr],
@@ -111,6 +122,7 @@ _RESTYPES = {
     "he_attention_plain_workspace_floats": c_i64,
     "he_ssm_state_floats": c_i64,
     "he_mlstm_state_floats": c_i64,
+    "he_delta_state_floats": c_i64,
     "he_gemm_plain_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
     "he_attention_decode_fused_workspace_floats": c_i64,

@@ -567,15 +567,17 @@ def qkv_rope_cache(q_out, kpool, vpool, qkv, q_cols: int, kv_cols: int, bias, po
 
 @_op("conv_state")
 def conv_state(out, x, taps, bias, state, positions, row_seq, seq_slot, seq_start, cu_seqlens,
-               rows: int, num_seqs: int, all_single: bool) -> None:
-    """out[rows, C] = silu(causal convolution per channel of x + bias), the taps' last column on the
+               rows: int, num_seqs: int, all_single: bool, act: bool = True) -> None:
+    """out[rows, C] = silu(causal convolution per channel of x + bias) (bias None: none; act False: the
+    convolution's sum as it is), the taps' last column on the
     row's own input; the inputs before a step's first row come from the sequence's row of `state`
     (uint8 [slots, bytes], fp32 [K-1][C] at its start), which is then moved on. x: a view [rows, C]
     of wider rows (unit stride along C)."""
     C, K = taps.shape
     _need(out, "out", x.dtype, (None, C))
     _need(taps, "taps")
-    _need(bias, "bias", taps.dtype, (C,))
+    if bias is not None:
+        _need(bias, "bias", taps.dtype, (C,))
     if x.dim() != 2 or x.shape[1] != C or x.stride(1) != 1 or x.shape[0] < rows or out.shape[0] < rows:
         raise ValueError("conv_state: x must be [rows, C] with unit stride along C")
     if state.dtype != torch.uint8 or state.dim() != 2 or state.stride(1) != 1:
@@ -588,10 +590,10 @@ def conv_state(out, x, taps, bias, state, positions, row_seq, seq_slot, seq_star
     if state.shape[1] < 4 * (K - 1) * C:
         raise ValueError("conv_state: the state rows are too short")
     L = _lib.load()
-    _lib.check(L.he_conv_state(out.data_ptr(), x.data_ptr(), x.stride(0), taps.data_ptr(), bias.data_ptr(),
+    _lib.check(L.he_conv_state(out.data_ptr(), x.data_ptr(), x.stride(0), taps.data_ptr(), _ptr(bias),
                                dtype_code(taps.dtype), state.data_ptr(), state.stride(0), positions.data_ptr(),
                                row_seq.data_ptr(), seq_slot.data_ptr(), seq_start.data_ptr(), cu_seqlens.data_ptr(),
-                               rows, num_seqs, C, K, int(all_single), dtype_code(x.dtype), _stream()))
+                               rows, num_seqs, C, K, int(all_single), int(act), dtype_code(x.dtype), _stream()))
 
 
 def ssm_state_floats(R: int, P: int, N: int) -> int:
@@ -635,7 +637,7 @@ def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float, gate_
     """out[rows, W] = (y * silu(z)), each of `parts` equal stretches of a row divided by its own root mean
     square, times weight. y fp32 [rows, W]; z a view [rows, W] of wider rows in out's dtype. gate_after: each
     stretch of y is divided by its own root mean square as it is, and the result is multiplied by weight,
-    sigmoid(z) and out_scale."""
+    sigmoid(z) and out_scale; gate_after "silu": by silu(z) in place of sigmoid(z)."""
     W = weight.shape[0]
     _need(out, "out", None, (None, W))
     _need(y, "y", torch.float32, (None, W))
@@ -646,11 +648,168 @@ def gated_group_norm(out, y, z, weight, rows: int, parts: int, eps: float, gate_
         raise ValueError("gated_group_norm: buffers smaller than the row count, or parts that do not divide the width")
     L = _lib.load()
     _lib.check(L.he_gated_group_norm(out.data_ptr(), y.data_ptr(), z.data_ptr(), z.stride(0), weight.data_ptr(),
-                                     dtype_code(weight.dtype), rows, W, parts, float(eps), int(gate_after),
+                                     dtype_code(weight.dtype), rows, W, parts, float(eps), 2 if gate_after == "silu" else int(bool(gate_after)),
                                      float(out_scale), dtype_code(out.dtype), _stream()))
 
 
 ACT_KINDS = {"relu2": 0, "gelu_tanh": 1, "silu": 2, "relu": 3}
+
+
+def delta_state_floats(H: int, d: int, e: int) -> int:
+    """Floats of a sequence's delta-rule state (the key dims padded to the lanes' shares)."""
+    return int(_lib.load().he_delta_state_floats(H, d, e))
+
+
+@_op("delta_scan")
+def delta_scan(y, q, k, v, ba, a_log, dt_bias, state, state_offset: int, cu_seqlens, seq_slot, rows: int,
+               num_seqs: int, H: int, G: int, d: int, e: int, q_scale: float, unit_eps: float) -> None:
+    """y (fp32 [rows, H e]) = the gated delta rule over q, k [rows, G d] and v [rows, H e] (views of rows of one
+    buffer, unit stride along the columns), ba (fp32 [rows, 2 H]: write strengths, then decay inputs, both before
+    their sigmoid / softplus) and per head a_log, dt_bias; the state [H][e][d'] lives at byte state_offset of a
+    sequence's row of `state` and is carried on."""
+    _need(y, "y", torch.float32, (None, H * e))
+    _need(ba, "ba", torch.float32, (None, 2 * H))
+    stride = q.stride(0)
+    for name, t, width in (("q", q, G * d), ("k", k, G * d), ("v", v, H * e)):
+        if not t.is_cuda or t.dtype != q.dtype or t.dim() != 2 or t.shape[1] != width or t.stride(1) != 1 \
+                or t.stride(0) != stride or t.shape[0] < rows:
+            raise ValueError(f"delta_scan: {name} must be a [rows, {width}] view of rows {stride} elements apart")
+    _need(a_log, "a_log", None, (H,))
+    _need(dt_bias, "dt_bias", a_log.dtype, (H,))
+    if y.shape[0] < rows or ba.shape[0] < rows:
+        raise ValueError("delta_scan: buffers smaller than the row count")
+    if state.dtype != torch.uint8 or state.dim() != 2 or state.stride(1) != 1 \
+            or state.shape[1] < state_offset + 4 * delta_state_floats(H, d, e):
+        raise ValueError("delta_scan: state must be uint8 [slots, bytes] with room for the heads' matrices")
+    _need(cu_seqlens, "cu_seqlens", torch.int32)
+    _need(seq_slot, "seq_slot", torch.int32)
+    if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs:
+        raise ValueError("delta_scan: metadata shorter than the step")
+    L = _lib.load()
+    _lib.check(L.he_delta_scan(y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, ba.data_ptr(),
+                               a_log.data_ptr(), dt_bias.data_ptr(), dtype_code(a_log.dtype), state.data_ptr(),
+                               state.stride(0), state_offset, cu_seqlens.data_ptr(), seq_slot.data_ptr(), rows, num_seqs,
+                               H, G, d, e, float(q_scale), float(unit_eps), dtype_code(q.dtype), _stream()))
+
+
+@_op("add_group_normed")
+def add_group_normed(resid_f32, delta, weight, groups: int, eps: float, delta_scale: float, out, rows: int, *,
+                     next_weight=None, next_groups: int = 1, next_eps: float = 0.0) -> None:
+    """resid += delta_scale * gn(delta), gn the RMS norm in `groups` equal consecutive parts of the row times weight
+    (delta None: nothing is added); then, with out, out = gn'(resid) by (next_weight, next_groups, next_eps), or resid
+    itself in out's dtype where next_weight is None."""
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    if delta is not None:
+        _need(delta, "delta", None, (None, D))
+        _need(weight, "weight", None, (D,))
+    if out is not None:
+        _need(out, "out", None, (None, D))
+    if next_weight is not None:
+        _need(next_weight, "next_weight", weight.dtype if delta is not None else None, (D,))
+    if resid_f32.shape[0] < rows or (delta is not None and delta.shape[0] < rows) or (out is not None and out.shape[0] < rows):
+        raise ValueError("add_group_normed: buffers smaller than the row count")
+    w = weight if delta is not None else next_weight
+    L = _lib.load()
+    _lib.check(L.he_add_group_normed(resid_f32.data_ptr(), _ptr(delta), dtype_code(delta.dtype) if delta is not None else F32,
+                                     _ptr(weight) if delta is not None else None, dtype_code(w.dtype) if w is not None else F32,
+                                     int(groups), float(eps), float(delta_scale), _ptr(out),
+                                     dtype_code(out.dtype) if out is not None else F32, _ptr(next_weight), int(next_groups),
+                                     float(next_eps), rows, D, _stream()))
+
+
+@_op("polynorm")
+def polynorm(out, x, numbers, rows: int, eps: float) -> None:
+    """out[r] = a N(z) + b N(z^2) + c N(z^3) + e over row r of x, powers element by element, N the division by the root
+    mean square (eps inside the root), numbers = (a, b, c, e). out may be x."""
+    W = x.shape[-1]
+    _need(x, "x", None, (None, W))
+    _need(out, "out", x.dtype, (None, W))
+    _need(numbers, "numbers", None, (4,))
+    if min(x.shape[0], out.shape[0]) < rows:
+        raise ValueError("polynorm: buffers smaller than the row count")
+    L = _lib.load()
+    _lib.check(L.he_polynorm(out.data_ptr(), x.data_ptr(), numbers.data_ptr(), dtype_code(numbers.dtype), rows, W,
+                             float(eps), dtype_code(x.dtype), _stream()))
+
+
+@_op("qk_head_norm")
+def qk_head_norm(out, x, q_weight, k_weight, H: int, G: int, d: int, eps: float, rows: int, copy_v: bool = False) -> None:
+    """x [rows, (H + G) d or wider]: every q head (the first H stretches of d) and every k head (the next G) is
+    divided by its own root mean square and multiplied by q_weight / k_weight [d], into the same columns of out
+    (which may be x); copy_v: the k heads as they were before the norm become the G stretches of out behind them (the
+    values are the keys)."""
+    for name, t, cols in (("x", x, (H + G) * d), ("out", out, (H + G + (G if copy_v else 0)) * d)):
+        if not t.is_cuda or t.dtype != x.dtype or t.dim() != 2 or t.stride(1) != 1 or t.shape[0] < rows or t.shape[1] < cols:
+            raise ValueError(f"qk_head_norm: {name} must be [rows, {cols} or wider] with unit stride along the columns")
+    _need(q_weight, "q_weight", None, (d,))
+    _need(k_weight, "k_weight", q_weight.dtype, (d,))
+    L = _lib.load()
+    _lib.check(L.he_qk_head_norm(out.data_ptr(), out.stride(0), x.data_ptr(), x.stride(0), q_weight.data_ptr(),
+                                 k_weight.data_ptr(), dtype_code(q_weight.dtype), H, G, d, float(eps), int(copy_v), rows,
+                                 dtype_code(x.dtype), _stream()))
+
+
+@_op("depth_mix")
+def depth_mix(resid_f32, kept_f32, coeffs, n: int, rows: int) -> None:
+    """kept[n - 1] = resid; resid = sum_{j < n} coeffs[j] * kept[j] (fp32, added in ascending j). kept: fp32
+    [n or more, rows of the step, D]; resid: fp32 [rows, D]."""
+    D = resid_f32.shape[-1]
+    _need(resid_f32, "resid", torch.float32)
+    _need(kept_f32, "kept", torch.float32)
+    _need(coeffs, "coeffs")
+    if kept_f32.dim() != 3 or kept_f32.shape[0] < n or kept_f32.shape[2] != D or kept_f32.shape[1] < rows \
+            or resid_f32.shape[0] < rows or coeffs.numel() < n or n < 1:
+        raise ValueError("depth_mix: kept must be [n or more, rows, D] and coeffs hold n numbers")
+    L = _lib.load()
+    _lib.check(L.he_depth_mix(resid_f32.data_ptr(), kept_f32.data_ptr(), kept_f32.stride(0), coeffs.data_ptr(),
+                              dtype_code(coeffs.dtype), n, rows * D, _stream()))
+
+
+@_op("gated_add")
+def gated_add(out, a, b, x, gate_weight, rows: int) -> None:
+    """out[r] = a[r] + sigmoid(x[r] . gate_weight) * b[r]; the dot product in fp32."""
+    D, Dx = a.shape[-1], x.shape[-1]
+    _need(a, "a", None, (None, D))
+    _need(b, "b", a.dtype, (None, D))
+    _need(out, "out", a.dtype, (None, D))
+    _need(x, "x", a.dtype, (None, Dx))
+    _need(gate_weight, "gate_weight")
+    if gate_weight.numel() != Dx or min(a.shape[0], b.shape[0], out.shape[0], x.shape[0]) < rows:
+        raise ValueError("gated_add: buffers smaller than the row count, or a gate of another width")
+    L = _lib.load()
+    _lib.check(L.he_gated_add(out.data_ptr(), a.data_ptr(), b.data_ptr(), x.data_ptr(), gate_weight.data_ptr(),
+                              dtype_code(gate_weight.dtype), rows, D, Dx, dtype_code(a.dtype), _stream()))
+
+
+@_op("head_product")
+def head_product(out, x, w, rows: int) -> None:
+    """out[r, h, :] = x[r, h, :] @ w[h] for views out [rows, H, N] and x [rows, H, K] (unit stride along the last
+    axis, any row and head strides) and w [H, K, N]; fp32 sums in ascending k."""
+    H, K, N = w.shape
+    _need(w, "w")
+    for name, t, last in (("x", x, K), ("out", out, N)):
+        if not t.is_cuda or t.dtype != x.dtype or t.dim() != 3 or t.shape[1] != H or t.shape[2] != last \
+                or t.stride(2) != 1 or t.shape[0] < rows:
+            raise ValueError(f"head_product: {name} must be a [rows, {H}, {last}] view with unit stride along the last axis")
+    L = _lib.load()
+    _lib.check(L.he_head_product(out.data_ptr(), out.stride(0), out.stride(1), x.data_ptr(), x.stride(0), x.stride(1),
+                                 w.data_ptr(), dtype_code(w.dtype), rows, H, K, N, dtype_code(x.dtype), _stream()))
+
+
+@_op("latent_pack")
+def latent_pack(qkv, q, down, rows: int, H: int, d: int, r: int, rank: int) -> None:
+    """qkv [rows, H (r + rank) + (r + rank) + rank]: head h's first r columns = the last r of q[row, h] (q [rows, H (d + r)]),
+    the key = [down[row, rank:rank + r] | down[row, :rank]], the value = down[row, :rank] (down: a view [rows, rank + r])."""
+    hd = r + rank
+    _need(qkv, "qkv", None, (None, (H + 1) * hd + rank))
+    _need(q, "q", qkv.dtype, (None, H * (d + r)))
+    if not down.is_cuda or down.dtype != qkv.dtype or down.dim() != 2 or down.shape[1] != rank + r or down.stride(1) != 1 \
+            or min(down.shape[0], q.shape[0], qkv.shape[0]) < rows:
+        raise ValueError("latent_pack: down must be a [rows, rank + r] view in qkv's dtype")
+    L = _lib.load()
+    _lib.check(L.he_latent_pack(qkv.data_ptr(), q.data_ptr(), down.data_ptr(), down.stride(0), rows, H, d, r, rank,
+                                dtype_code(qkv.dtype), _stream()))
 
 
 @_op("add_normed")
@@ -791,27 +950,28 @@ def mlstm_scan(y, q, k, v, gates, state, state_offset: int, cu_seqlens, seq_slot
 
 @_op("route_tokens")
 def route_tokens(dense, ids, weights, logits, correction, rows: int, real: int, groups: int, keep: int,
-                 top: int, scale: float, *, x=None, router=None) -> None:
+                 top: int, scale: float, *, x=None, router=None, normalize: bool = False) -> None:
     """The choice of `top` of E router outputs per row (logits fp32 [rows, E]; or logits None and the kernel
     forms them in fp32 from the rows x [rows, D] and the router's matrix, fp32 [E, D]): softmax scores s, the
     choice on s + correction inside the `keep` best of `groups` equal groups, weights s * scale. dense (fp32
     [rows, real + 1]): each expert's weight or 0, the outputs from `real` on added up in the last column;
-    ids (int32) and weights (fp32) [rows, top]: the chosen outputs."""
+    ids (int32) and weights (fp32) [rows, top]: the chosen outputs. normalize: the chosen outputs' weights are divided
+    by their sum (times scale): the softmax over the chosen logits alone."""
     if logits is None:
         E, D = router.shape
         _need(router, "router", torch.float32)
         _need(x, "x", None, (None, D))
         if x.shape[0] < rows:
             raise ValueError("route_tokens: x has fewer rows than the step")
-        return _route(dense, ids, weights, None, x, router, correction, rows, E, real, groups, keep, top, scale)
+        return _route(dense, ids, weights, None, x, router, correction, rows, E, real, groups, keep, top, scale, normalize)
     E = logits.shape[-1]
     _need(logits, "logits", torch.float32, (None, E))
     if logits.shape[0] < rows:
         raise ValueError("route_tokens: buffers smaller than the row count")
-    _route(dense, ids, weights, logits, None, None, correction, rows, E, real, groups, keep, top, scale)
+    _route(dense, ids, weights, logits, None, None, correction, rows, E, real, groups, keep, top, scale, normalize)
 
 
-def _route(dense, ids, weights, logits, x, router, correction, rows, E, real, groups, keep, top, scale) -> None:
+def _route(dense, ids, weights, logits, x, router, correction, rows, E, real, groups, keep, top, scale, normalize=False) -> None:
     _need(dense, "dense", torch.float32, (None, real + 1))
     _need(ids, "ids", torch.int32, (None, top))
     _need(weights, "weights", torch.float32, (None, top))
@@ -824,7 +984,7 @@ def _route(dense, ids, weights, logits, x, router, correction, rows, E, real, gr
                                  _ptr(x), dtype_code(x.dtype) if x is not None else F32, _ptr(router),
                                  router.shape[1] if router is not None else 0,
                                  _ptr(correction), dtype_code(correction.dtype) if correction is not None else F32,
-                                 rows, E, real, groups, keep, top, float(scale), _stream()))
+                                 rows, E, real, groups, keep, top, float(scale), int(normalize), _stream()))
 
 
 @_op("routed_act")
@@ -899,18 +1059,21 @@ def _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd):
 @_op("attention_plain")
 def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
                     H: int, KVH: int, hd: int, window: int, scale: float, most_keys: int = 0,
-                    workspace=None, *, chunk: int = 0, sinks=None, gate=None) -> None:
+                    workspace=None, *, chunk: int = 0, sinks=None, gate=None, slopes=None) -> None:
     """most_keys: a bound on the keys any sequence holds after the step, and workspace: fp32, of
     attention_plain_workspace_floats elements or more: the pages of a query then run in parallel
     (a step of few queries over many keys); the result is the same bit for bit without them.
     chunk > 0: a query sees the keys of its own chunk of so many positions only (counted from
     position 0). sinks [H]: a number a head that joins the softmax's denominator as exp(sink).
     gate: a view [rows, H] of q's dtype (unit stride along heads, any row stride): the head's output
-    is multiplied by sigmoid(gate)."""
+    is multiplied by sigmoid(gate). slopes (fp32 [H]): the score of key j for the query at p loses
+    slopes[h] * (p - j)."""
     _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
     gate_ptr, gate_stride = _gate_view(gate, q, rows, H)
     if sinks is not None:
         _need(sinks, "sinks", shape=(H,))
+    if slopes is not None:
+        _need(slopes, "slopes", torch.float32, (H,))
     if workspace is not None:
         _need(workspace, "workspace", torch.float32)
     for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
@@ -924,7 +1087,7 @@ def attention_plain(out, q, kpool, vpool, positions, row_seq, seq_slot, page_tab
         kpool.shape[0], rows, H, KVH, hd, window, int(chunk), float(scale), _ptr(sinks),
         dtype_code(sinks.dtype) if sinks is not None else F32, gate_ptr, gate_stride,
         dtype_code(q.dtype), int(most_keys),
-        _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()))
+        _ptr(workspace), workspace.numel() if workspace is not None else 0, _ptr(slopes), _stream()))
 
 
 def _gate_view(gate, q, rows: int, H: int):

@@ -1,6 +1,6 @@
 """Parts a layer is put together from, and their registries."""
-from . import (attention, block, embedding, matrix_memory, mlp, norm, parallel, rotary, routed, state_space,  # noqa: F401
-               token_input)  # noqa: F401  (register the built-in parts)
+from . import (attention, block, delta_rule, embedding, latent_attention, matrix_memory, mlp, norm, parallel, rotary,  # noqa: F401
+               routed, state_space, token_input)  # noqa: F401  (register the built-in parts)
 from .base import (Block, BuildEnv, FeedForward, KVNeed, LayerCache, LayerSpec, Mixer, ModelSpec,
                    Norm, Part, PartSpec, PositionEncoding, ResidualStream, ScheduleEntry,
                    StepContext, TensorSpec, build_part, param, register_part, registered)

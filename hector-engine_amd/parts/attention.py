@@ -27,7 +27,17 @@ Options of the same part, each off unless its parameter says otherwise:
               every value of every head (tensor `gate`); its rows ride behind q||k||v likewise.
   qk_norm     "projection": q (all heads' rows of a token at once) is divided by its root mean square
               (eps `qk_norm_eps`) and multiplied by a stored vector of that size, k likewise; after the
-              bias and before the position encoding.
+              bias and before the position encoding. "head": every head of q is divided by its own root
+              mean square and multiplied by one stored vector of head_dim that all heads share, every
+              head of k likewise with a second vector.
+  conv_taps   K > 0: q and k pass a causal convolution per channel over the last K projected rows of the
+              sequence (tensors `q_conv`, `k_conv`, [channels, K], the last column on the row's own
+              input, zeros before the sequence's start, no bias), directly behind the projection and
+              before the norm; the sequence carries the last K - 1 projected rows in its state.
+  values      "keys": there is no value projection; a kv head's value is its key as it stands before
+              the q/k norm (behind the convolution). value_dim must equal head_dim.
+  distance_slope_span  s > 0: the score of key j for the query at position i loses slope_h * (i - j), with
+              slope_h = 2^(-s (h + 1) / H) for head h.
   q_temp      {coef, every}: the q of position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1).
   score_maps  2: differential attention. A head has two queries and a kv head two keys (in the q and k
               matrices a head's rows for map 1 stand in front of its rows for map 2); the two maps are
@@ -38,7 +48,7 @@ Options of the same part, each off unless its parameter says otherwise:
               so that the heads of one (kv head, map) are neighbours, and the value rows of a kv head
               stand once for each of its maps; ops.diff_heads then joins the pairs.
   names       the suffixes of its tensors (q, k, v, o, q_bias, k_bias, v_bias, o_bias, sinks, gate,
-              lq1, lk1, lq2, lk2, q_norm, k_norm).
+              lq1, lk1, lq2, lk2, q_norm, k_norm, q_conv, k_conv).
 """
 from __future__ import annotations
 
@@ -54,7 +64,7 @@ from .base import (BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, PieceRows, Ste
 _NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
           "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
           "sinks": "sinks", "gate": "gate.weight", "lq1": "lambda_q1", "lk1": "lambda_k1", "lq2": "lambda_q2",
-          "lk2": "lambda_k2", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+          "lk2": "lambda_k2", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "q_conv": "q_conv.weight", "k_conv": "k_conv.weight"}
 from .linear import Linear
 
 
@@ -101,6 +111,11 @@ class Attention(Mixer):
         self.qk_norm = param(params, "qk_norm", str, "")
         self.qk_norm_eps = param(params, "qk_norm_eps", float, 1e-6)
         self.q_norm_w = self.k_norm_w = None
+        self.conv_taps = param(params, "conv_taps", int, 0)
+        self.values_are_keys = param(params, "values", str, "projection") == "keys"
+        self.slope_span = param(params, "distance_slope_span", float, 0.0)
+        self.slopes: torch.Tensor | None = None
+        self.taps = None
         self.maps = param(params, "score_maps", int, 1)
         self.diff = param(params, "diff", float, 0.0)
         self.diff_eps = param(params, "diff_eps", float, 1e-6)
@@ -111,8 +126,17 @@ class Attention(Mixer):
             raise ValueError(f"attention: score_maps {self.maps} must be 1 or 2 (and 2 goes without gates and q/k norms)")
         if self.head_gate and self.out_gate:
             raise ValueError("attention: head_gate and out_gate exclude each other")
-        if self.qk_norm not in ("", "projection"):
+        if self.qk_norm not in ("", "projection", "head"):
             raise ValueError(f"attention: unknown qk_norm '{self.qk_norm}'")
+        if param(params, "values", str, "projection") not in ("projection", "keys"):
+            raise ValueError(f"attention: unknown values '{params['values']}'")
+        if self.conv_taps < 0 or self.slope_span < 0:
+            raise ValueError("attention: conv_taps and distance_slope_span must not be negative")
+        if (self.conv_taps or self.values_are_keys) and (self.qkv_bias or self.maps > 1 or self.head_gate or self.out_gate
+                                                         or not self.kv_projection):
+            raise ValueError("attention: conv_taps and values 'keys' go without biases, gates, score maps and shared caches")
+        if self.values_are_keys and self.vd != self.hd:
+            raise ValueError(f"attention: values that are the keys are head_dim {self.hd} wide, not {self.vd}")
         if self.has_sinks and self.sink_value is not None:
             raise ValueError("attention: stored sinks and sink_value exclude each other")
         if self.q_temp is not None and self.q_temp[1] <= 0:
@@ -138,15 +162,21 @@ class Attention(Mixer):
         self.o_proj: Linear | None = None
         self._chosen: dict[tuple, routes.Route] = {}      # (all one-token, dtype) -> route, for one version of the table
         self._chosen_version = -1
-        self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0   # else the plain kernel
+        # else the plain kernel (which alone takes the distance slopes)
+        self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0 and not self.slope_span
         # what the fused one-token kernel and the kernels without these options do not take
         self.extras = self.chunk > 0 or self.has_sinks or self.head_gate or self.maps > 1 or self.q_temp is not None \
-            or self.out_gate or self.sink_value is not None or bool(self.qk_norm)
+            or self.out_gate or self.sink_value is not None or bool(self.qk_norm) or self.conv_taps > 0 \
+            or self.values_are_keys or self.slope_span > 0
         # rows of the gate's matrix behind q||k||v: one a head, or one for every value of every head
         self.gate_rows = self.H if self.head_gate else self.H * self.vd if self.out_gate else 0
 
     def children(self):
         return [self.position]
+
+    def state_bytes(self) -> int:
+        # the last K - 1 projected q and k rows of the sequence, fp32
+        return 4 * (self.conv_taps - 1) * (self.Hk + self.KVHk) * self.hd if self.conv_taps > 1 else 0
 
     def kv_need(self):
         # pages in the order the attention kernels read their operands
@@ -159,7 +189,11 @@ class Attention(Mixer):
                  n["o"]: TensorSpec((self.hidden, self.H * vd))}
         if self.kv_projection:
             specs[n["k"]] = TensorSpec((self.KVHk * hd, self.hidden))
-            specs[n["v"]] = TensorSpec((self.KVH * vd, self.hidden))
+            if not self.values_are_keys:
+                specs[n["v"]] = TensorSpec((self.KVH * vd, self.hidden))
+        if self.conv_taps:
+            specs[n["q_conv"]] = TensorSpec((self.H * hd, self.conv_taps), ("normal", 0.4))
+            specs[n["k_conv"]] = TensorSpec((self.KVH * hd, self.conv_taps), ("normal", 0.4))
         if self.qkv_bias:
             specs[n["q_bias"]] = TensorSpec((self.Hk * hd,))
             if self.kv_projection:
@@ -175,15 +209,16 @@ class Attention(Mixer):
         if self.gate_rows:
             specs[n["gate"]] = TensorSpec((self.gate_rows, self.hidden))
         if self.qk_norm:
-            specs[n["q_norm"]] = TensorSpec((self.H * hd,), ("gain", 1.0, 0.1))
+            per_head = self.qk_norm == "head"
+            specs[n["q_norm"]] = TensorSpec((hd if per_head else self.H * hd,), ("gain", 1.0, 0.1))
             if self.kv_projection:
-                specs[n["k_norm"]] = TensorSpec((self.KVH * hd,), ("gain", 1.0, 0.1))
+                specs[n["k_norm"]] = TensorSpec((hd if per_head else self.KVH * hd,), ("gain", 1.0, 0.1))
         specs.update(self.position.tensor_specs())
         return specs
 
     def bind(self, tensors):
         p, n = self.prefix, self._names
-        names = ["q"] + (["k", "v"] if self.kv_projection else [])
+        names = ["q"] + ((["k"] if self.values_are_keys else ["k", "v"]) if self.kv_projection else [])
         ws = [self._by_map(x, tensors.pop(n[x])) for x in names]
         gate_w = tensors.pop(n["gate"]) if self.gate_rows else None
         if gate_w is not None:
@@ -234,6 +269,12 @@ class Attention(Mixer):
         if self.qk_norm:
             self.q_norm_w = tensors[n["q_norm"]]
             self.k_norm_w = tensors[n["k_norm"]] if self.kv_projection else None
+        if self.conv_taps:
+            self.taps = torch.cat([tensors[n["q_conv"]], tensors[n["k_conv"]]], 0).contiguous()
+            self._no_state = torch.zeros((1, 16), dtype=torch.uint8, device=wo.device)
+        if self.slope_span:
+            h = torch.arange(1, self.H + 1, dtype=torch.float64)
+            self.slopes = torch.exp2(-self.slope_span * h / self.H).to(torch.float32).to(wo.device)
         self.position.bind(tensors)
 
     def _by_map(self, which: str, t: torch.Tensor) -> torch.Tensor:
@@ -317,7 +358,12 @@ class Attention(Mixer):
         # any other encoding sees q and k with their bias already added.
         fused_bias = not self.position.custom and not self.qk_norm
         qkv = proj(x, rows, ctx, use_bias=not fused_bias)
-        if self.qk_norm:
+        if self.conv_taps or self.values_are_keys:
+            qkv = self._conv_norm_rows(qkv, ctx, cache)
+        elif self.qk_norm == "head":
+            ops.qk_head_norm(qkv, qkv, self.q_norm_w, self.k_norm_w if writes else self.q_norm_w, H, KVH if writes else 0,
+                             hd, self.qk_norm_eps, rows)
+        elif self.qk_norm:
             # each token's q (all heads at once), and its k, by a root mean square of their own, in place
             wide = qkv.stride(0)
             if writes:
@@ -342,6 +388,34 @@ class Attention(Mixer):
             gate = qkv[:rows, at:at + self.gate_rows]
         return q, gate
 
+    def _conv_norm_rows(self, qk, ctx: StepContext, cache: LayerCache):
+        """The rows [q | k | v] the cache-write kernel reads, from the projected [q | k]: the convolution over
+        each sequence's rows (with the rows it carries), then the heads' norm; the keys as they leave the
+        convolution are the values."""
+        rows, H, KVH, hd = ctx.rows, self.H, self.KVH, self.hd
+        C = (H + KVH) * hd
+        if self.conv_taps:
+            if self.conv_taps > 1 and cache.state is None:
+                raise RuntimeError(f"{self.prefix}: a convolution over the rows needs its row of the state area")
+            conv = ctx.alloc((rows, C))
+            state = cache.state if cache.state is not None else self._no_state     # one tap carries nothing
+            ops.conv_state(conv, qk[:, :C], self.taps, None, state, ctx.positions, ctx.row_seq, ctx.seq_slot,
+                           ctx.seq_start, ctx.cu_seqlens, rows, ctx.num_seqs, ctx.all_single, act=False)
+            qk = conv
+        if not self.values_are_keys:
+            if self.qk_norm == "head":
+                ops.qk_head_norm(qk, qk, self.q_norm_w, self.k_norm_w, H, KVH, hd, self.qk_norm_eps, rows)
+            elif self.qk_norm:
+                raise ValueError(f"{self.prefix}: a convolution goes with the heads' own norm or none")
+            return qk
+        out = ctx.alloc((rows, C + KVH * hd))
+        if self.qk_norm == "head":
+            ops.qk_head_norm(out, qk, self.q_norm_w, self.k_norm_w, H, KVH, hd, self.qk_norm_eps, rows, copy_v=True)
+        else:
+            out[:rows, :C].copy_(qk[:rows, :C])
+            out[:rows, C:].copy_(qk[:rows, H * hd:C])
+        return out
+
     def _run_plain(self, x, ctx: StepContext, cache: LayerCache):
         """The plain kernel: one fixed order per (query, head), in the precision of the cache."""
         rows, H, KVH, hd = ctx.rows, self.Hk, self.KVHk, self.pd
@@ -351,7 +425,8 @@ class Attention(Mixer):
         ws = ctx.alloc((floats,), torch.float32) if floats else None
         ops.attention_plain(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                             ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                            self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+                            self.scale, ctx.most_keys, ws, chunk=self.chunk, sinks=self.sinks,
+                            gate=gate if self.head_gate else None, slopes=self.slopes)
         return self._project(out, rows, ctx, gate)
 
     def _run_mfma_one_token(self, x, ctx: StepContext, cache: LayerCache):

@@ -76,6 +76,10 @@ class ModelSpec:
     # full names of tensors a model folder may hold although the model does not use them
     # (an output matrix stored beside the embedding it is tied to)
     unused_tensors: frozenset = frozenset()
+    # depth mix: one full tensor name per schedule entry, or None. With X_0 the embedding's output and X_(e+1)
+    # the stream as run e leaves it, what goes on to the next run (after the last one: to the final norm) is
+    # sum over j <= e + 1 of c_e[j] * X_j, with c_e the e + 2 numbers of entry e's tensor.
+    depth_mix: list | None = None
 
 
 PAGE_TOKENS = 64     # tokens of a cache page

@@ -6,7 +6,10 @@ rows, done by the last product of the mixer / feed-forward, which then also prep
 the rows of the norm that follows (parts.base.ResidualSink).
 
 residual_scale m (1 unless given): x = x + m * mixer(norm1(x)); x = x + m * feed_forward(norm2(x)).
-A layer without a feed-forward (feed_forward None) is the first line alone."""
+A layer without a feed-forward (feed_forward None) is the first line alone.
+
+The "post_norm" block norms what a branch returns and nothing it reads:
+    x = x + m * norm1(mixer(x));  x = x + m * norm2(feed_forward(x))."""
 from __future__ import annotations
 
 import torch
@@ -171,3 +174,76 @@ class SandwichNormBlock(Block):
             n = self._join(stream, delta, post, after, ctx)
         if after is not None and n is not None:
             stream.ready = (after, n)
+
+
+@register_part("block", "post_norm")
+class PostNormBlock(Block):
+    """A layer whose branches read the stream itself (in the activation dtype) and are normed on their way
+    back into it:  x = x + m * norm1(mixer(x));  x = x + m * norm2(feed_forward(x)), with m = residual_scale
+    (1 unless given). A layer without a feed-forward is the first line alone.
+
+    Each sum is one launch where the norm has add_normed_delta (the grouped RMS norm): the branch output is
+    normed and added in fp32, and the same launch writes the new stream's rows in the activation dtype for the
+    branch that reads them next. Other norms go through their own add_norm on a 32-bit copy of the branch output.
+    names: mixer_norm, mixer, feed_forward_norm, feed_forward (suffixes of the parts' prefixes)."""
+
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        names = param(params, "names", dict)
+        self.mixer_norm = build_part("norm", param(params, "mixer_norm", PartSpec),
+                                     prefix + names["mixer_norm"] + ".", env)
+        self.mixer = build_part("mixer", param(params, "mixer", PartSpec), prefix + names["mixer"] + ".", env)
+        self.residual_scale = param(params, "residual_scale", float, 1.0)
+        self.ff_norm = self.feed_forward = None
+        if param(params, "feed_forward", PartSpec, None) is not None:
+            self.ff_norm = build_part("norm", param(params, "feed_forward_norm", PartSpec),
+                                      prefix + names["feed_forward_norm"] + ".", env)
+            self.feed_forward = build_part("feed_forward", param(params, "feed_forward", PartSpec),
+                                           prefix + names["feed_forward"] + ".", env)
+
+    def children(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward) if p is not None]
+
+    def tensor_specs(self):
+        specs = {}
+        for c in self.children():
+            specs.update(c.tensor_specs())
+        return specs
+
+    def bind(self, tensors):
+        for c in self.children():
+            c.bind(tensors)
+
+    def _rows(self, stream: ResidualStream, ctx: StepContext):
+        """The stream as it stands, in the activation dtype."""
+        from ..kernels import ops
+        resid = stream.materialize(ctx)
+        out = ctx.alloc((stream.rows, resid.shape[-1]))
+        ops.add_group_normed(resid, None, None, 1, 0.0, 1.0, out, stream.rows)
+        return out
+
+    def _join(self, stream: ResidualStream, delta, norm, want_rows: bool, ctx: StepContext):
+        """stream += m * norm(delta); returns the new stream's rows in the activation dtype when asked."""
+        from ..kernels import ops
+        rows = stream.rows
+        resid = stream.materialize(ctx)
+        stream.prepared = stream.ready = None
+        out = ctx.alloc((rows, resid.shape[-1])) if want_rows else None
+        if hasattr(norm, "add_normed_delta"):
+            norm.add_normed_delta(resid, delta, rows, self.residual_scale, out)
+            return out
+        copy = ctx.alloc((rows, resid.shape[-1]), torch.float32)
+        copy[:rows].copy_(delta[:rows])
+        normed = norm.add_norm(copy, None, rows, ctx)
+        ops.residual_add(resid, normed, rows, self.residual_scale)
+        if want_rows:
+            out[:rows].copy_(resid[:rows])
+        return out
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: LayerCache) -> None:
+        ctx.sink = None
+        delta = self.mixer.forward(self._rows(stream, ctx), ctx, cache)
+        x = self._join(stream, delta, self.mixer_norm, self.feed_forward is not None, ctx)
+        if self.feed_forward is not None:
+            delta = self.feed_forward.forward(x, ctx)
+            self._join(stream, delta, self.ff_norm, False, ctx)

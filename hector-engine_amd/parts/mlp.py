@@ -98,7 +98,10 @@ class GatedMLP(FeedForward):
 @register_part("feed_forward", "dense_mlp")
 class DenseMLP(FeedForward):
     """Feed-forward without a gate: d = act(x Wu^T) Wd^T, no biases. activation: "relu2" (the square of
-    relu), "gelu_tanh", "silu" or "relu". names: the suffixes of its tensors (up, down)."""
+    relu), "gelu_tanh", "silu" or "relu", element by element; or "polynorm", over a token's whole vector z of
+    intermediate values: a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, N the division by the root
+    mean square (eps `eps` inside the root), (a, b, c, e) the four stored numbers of the tensor `act`.
+    names: the suffixes of its tensors (up, down, act)."""
 
     accepts_normed_rows = True
 
@@ -107,28 +110,41 @@ class DenseMLP(FeedForward):
         self.hidden = param(params, "hidden_size", int)
         self.inter = param(params, "intermediate_size", int)
         self.act = param(params, "activation", str, "relu2")
-        if self.act not in ops.ACT_KINDS:
-            raise ValueError(f"dense_mlp: unsupported activation '{self.act}', have {sorted(ops.ACT_KINDS)}")
+        if self.act not in ops.ACT_KINDS and self.act != "polynorm":
+            raise ValueError(f"dense_mlp: unsupported activation '{self.act}', have {sorted(ops.ACT_KINDS) + ['polynorm']}")
+        self.eps = param(params, "eps", float, 1e-6)
+        self.numbers = None
         names = param(params, "names", dict, {})
         self._names = {k: tensor_name(prefix, names, k, d) for k, d in
-                       (("up", "up_proj.weight"), ("down", "down_proj.weight"))}
+                       (("up", "up_proj.weight"), ("down", "down_proj.weight"), ("act", "act.weight"))}
         self.up: Linear | None = None
         self.down: Linear | None = None
 
     def tensor_specs(self):
         n = self._names
-        return {n["up"]: TensorSpec((self.inter, self.hidden)), n["down"]: TensorSpec((self.hidden, self.inter))}
+        specs = {n["up"]: TensorSpec((self.inter, self.hidden)), n["down"]: TensorSpec((self.hidden, self.inter))}
+        if self.act == "polynorm":
+            specs[n["act"]] = TensorSpec((4,), ("gain", 0.3, 0.2))
+        return specs
 
     def bind(self, tensors):
         n = self._names
         self.up = Linear(tensors[n["up"]])
         self.down = Linear(tensors[n["down"]])
+        if self.act == "polynorm":
+            self.numbers = tensors[n["act"]]
+
+    def _activate(self, h, rows: int) -> None:
+        if self.act == "polynorm":
+            ops.polynorm(h, h, self.numbers, rows, self.eps)
+        else:
+            ops.unary_act(h, h, rows, self.act)
 
     def forward(self, x, ctx: StepContext):
         rows = ctx.rows
         if rows <= _ROW_CHUNK:
             h = self.up(x, rows, ctx)
-            ops.unary_act(h, h, rows, self.act)
+            self._activate(h, rows)
             return self.down(h, rows, ctx, sink=ctx.take_sink())
         if not isinstance(x, torch.Tensor):
             x = x.tensor(ctx)
@@ -137,7 +153,7 @@ class DenseMLP(FeedForward):
             n = min(_ROW_CHUNK, rows - r0)
             turn = ctx.scratch.mark()
             h = self.up(x[r0:r0 + n], n, ctx)
-            ops.unary_act(h, h, n, self.act)
+            self._activate(h, n)
             self.down(h, n, ctx, out=out[r0:r0 + n])
             ctx.scratch.release(turn)
         return out

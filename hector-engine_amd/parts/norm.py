@@ -72,3 +72,40 @@ class DynamicTanh(Norm):
         out = ctx.alloc((rows, self.size)) if want_out else None
         ops.add_dyt(resid, delta, self.weight, self.bias, self.alpha, out, rows, delta_scale)
         return out
+
+
+@register_part("norm", "group_rmsnorm")
+class GroupRMSNorm(Norm):
+    """RMS norm in groups: the vector is cut into `groups` equal consecutive parts, each is divided by its own
+    sqrt(mean(part^2) + eps), and the whole is multiplied by weight. No pair of products carries it (a row has
+    several scales). names: the suffix of its tensor (weight)."""
+
+    def __init__(self, params: dict, prefix: str, env: BuildEnv):
+        super().__init__(prefix, env)
+        self.size = param(params, "size", int)
+        self.groups = param(params, "groups", int, 1)
+        self.eps = param(params, "eps", float)
+        if self.groups <= 0 or self.size % self.groups:
+            raise ValueError(f"group_rmsnorm: {self.groups} groups do not divide the size {self.size}")
+        self._name = tensor_name(prefix, param(params, "names", dict, {}), "weight", "weight")
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return {self._name: TensorSpec((self.size,), ("gain", 1.0, 0.1))}
+
+    def bind(self, tensors):
+        self.weight = tensors[self._name]
+
+    def add_norm(self, resid, delta, rows, ctx: StepContext, want_out: bool = True, delta_scale: float = 1.0):
+        if delta is not None:
+            ops.residual_add(resid, delta, rows, delta_scale)
+        if not want_out:
+            return None
+        out = ctx.alloc((rows, self.size))
+        ops.add_group_normed(resid, None, None, 1, 0.0, 1.0, out, rows, next_weight=self.weight,
+                             next_groups=self.groups, next_eps=self.eps)
+        return out
+
+    def add_normed_delta(self, resid, delta, rows: int, scale: float, out) -> None:
+        """resid += scale * norm(delta); out (or None) receives the new rows of resid in its own dtype."""
+        ops.add_group_normed(resid, delta, self.weight, self.groups, self.eps, scale, out, rows)

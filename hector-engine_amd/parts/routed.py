@@ -19,6 +19,10 @@ product with the down matrices side by side (and an identity block) adds everyth
 has the same launches whatever the tokens choose, so it replays as a graph, and a token's sums do
 not depend on the rest of the batch. A bfloat16 step of so few rows that they cannot choose more than
 half of the experts reads only the chosen experts' rows of the same matrices (ops.chosen_experts).
+Options: `normalize` divides the chosen outputs' weights by their sum (the softmax over the chosen logits
+alone; the choice itself is the same, the softmax being monotone); `shared` = {"feed_forward": PartSpec, "name":
+suffix of its prefix, "gate": suffix of a stored vector of hidden_size or None} adds an expert that every token
+uses, out += sigmoid(gate . n) * shared(n) (gate None: out += shared(n)), the dot product in fp32.
 names: the suffixes of its tensors (router, correction; expert e's are 'e<e>.' + gate / up / down).
 """
 from __future__ import annotations
@@ -26,7 +30,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import BuildEnv, FeedForward, StepContext, TensorSpec, param, register_part, tensor_name
+from .base import BuildEnv, FeedForward, PartSpec, StepContext, TensorSpec, build_part, param, register_part, tensor_name
 from .linear import Linear
 
 # rows whose gate and up columns are held at once in a long prompt step
@@ -46,6 +50,13 @@ class RoutedExperts(FeedForward):
         self.groups = param(params, "groups", int, 1)
         self.keep = param(params, "keep_groups", int, self.groups)
         self.has_correction = param(params, "correction", bool, True)
+        self.normalize = param(params, "normalize", bool, False)
+        shared = param(params, "shared", dict, None)
+        self.shared = self.shared_gate = self._shared_gate = None
+        if shared:
+            self.shared = build_part("feed_forward", shared["feed_forward"], prefix + shared.get("name", "shared") + ".", env)
+            if shared.get("gate"):
+                self._shared_gate = prefix + shared.get("name", "shared") + "." + shared["gate"]
         self.limit = param(params, "limit", float, 0.0)
         self.alpha = param(params, "alpha", float, 1.702 if self.limit > 0 else 1.0)
         self.up_shift = param(params, "up_shift", float, 1.0 if self.limit > 0 else 0.0)
@@ -80,7 +91,14 @@ class RoutedExperts(FeedForward):
             specs[self._name(e, "gate")] = TensorSpec((self.inter, self.hidden))
             specs[self._name(e, "up")] = TensorSpec((self.inter, self.hidden))
             specs[self._name(e, "down")] = TensorSpec((self.hidden, self.inter))
+        if self.shared is not None:
+            specs.update(self.shared.tensor_specs())
+        if self._shared_gate:
+            specs[self._shared_gate] = TensorSpec((1, self.hidden))
         return specs
+
+    def children(self):
+        return [self.shared] if self.shared is not None else []
 
     def bind(self, tensors):
         # the router's sums are 32-bit whatever the run's precision: its matrix is kept in float32
@@ -97,6 +115,10 @@ class RoutedExperts(FeedForward):
             downs.append(torch.eye(self.hidden, dtype=downs[0].dtype, device=downs[0].device))
         self.gate_up = Linear(torch.cat(gu, 0).contiguous())
         self.down = Linear(torch.cat(downs, 1).contiguous())
+        if self.shared is not None:
+            self.shared.bind(tensors)
+        if self._shared_gate:
+            self.shared_gate = tensors[self._shared_gate].reshape(-1).contiguous()
 
     def _few_rows(self, rows: int, x, ctx: StepContext) -> bool:
         """Whether the step runs through the chosen experts alone (kernels.ops.chosen_experts): bfloat16 with the
@@ -106,13 +128,26 @@ class RoutedExperts(FeedForward):
                 and self.inter % 8 == 0 and self.hidden % 8 == 0 and 2 * rows * self.top <= self.real)
 
     def forward(self, x, ctx: StepContext):
+        if self.shared is None:
+            return self._routed(x, ctx, True)
+        rows = ctx.rows
+        routed = self._routed(x, ctx, False)
+        common = self.shared.forward(x, ctx)
+        out = ctx.alloc((rows, self.hidden))
+        if self.shared_gate is not None:
+            ops.gated_add(out, routed, common, x, self.shared_gate, rows)
+        else:
+            ops.scaled_sum(out, routed, common, rows, 1.0, 1.0)
+        return out
+
+    def _routed(self, x, ctx: StepContext, may_sink: bool):
         rows, real, I = ctx.rows, self.real, self.inter
         dense = ctx.alloc((rows, real + 1), torch.float32)
         ids = ctx.alloc((rows, self.top), torch.int32)
         weights = ctx.alloc((rows, self.top), torch.float32)
         # the router's product (fp32 sums over the rows as they are) and the choice, one launch
         ops.route_tokens(dense, ids, weights, None, self.correction, rows, real, self.groups, self.keep,
-                         self.top, self.scale, x=x, router=self.router)
+                         self.top, self.scale, x=x, router=self.router, normalize=self.normalize)
         cols = real * I + (self.hidden if self.identity else 0)
         act = {"alpha": self.alpha, "limit": self.limit, "up_shift": self.up_shift}
         if self._few_rows(rows, x, ctx):
@@ -125,7 +160,7 @@ class RoutedExperts(FeedForward):
             gu = self.gate_up(x, rows, ctx)
             h = ctx.alloc((rows, cols))
             ops.routed_act(h, gu, dense, x if self.identity else None, rows, real, I, **act)
-            return self.down(h, rows, ctx, sink=ctx.take_sink())
+            return self.down(h, rows, ctx, sink=ctx.take_sink() if may_sink else None)
         out = ctx.alloc((rows, self.hidden))
         for r0 in range(0, rows, _ROW_CHUNK):
             n = min(_ROW_CHUNK, rows - r0)
