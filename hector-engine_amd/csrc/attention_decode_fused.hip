@@ -341,6 +341,8 @@ __global__ __launch_bounds__(512) void attention_decode_fused_kernel(
   for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   st.m = -INFINITY;
   st.l = 0.f;
+  st.bias = 0.f;
+  st.pos = 0;
   if (has_keys) {
     bf16x8 qf[KS];
     rotate_q<NT>(qf, qx, lg, sn, c);

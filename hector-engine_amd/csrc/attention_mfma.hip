@@ -30,7 +30,7 @@
 // ------------------------------------------------------------------ prefill
 // grid (ceil(max_q_len / 64), H, num_seqs), 256 threads: wave w takes the 16
 // queries q0 = 64*blockIdx.x + 16*w of the sequence.
-template <int NT>
+template <int NT, bool BIAS>
 __global__ __launch_bounds__(256) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
     const uint16_t* __restrict__ kpool, const uint16_t* __restrict__ vpool,
@@ -65,6 +65,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   st.m = -INFINITY;
   st.l = 0.f;
+  st.bias = BIAS ? ex.slopes[h] / scale : 0.f;
+  st.pos = pos;
 
   const int last_pos = start + min(q0 + 15, q_len - 1);
   const int first_pos = start + q0;
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const bool full_tile = q0 + 15 < q_len;
   const int clear_lo = attn_first(last_pos, window, ex.chunk);
   const int clear_hi = full_tile ? first_pos : -1;
-  attend_range<NT, true>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
+  attend_range<NT, true, BIAS>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, tile_lo & ~31,
                    (last_pos & ~31) + 32, lo, hi, clear_lo, clear_hi, scale * 1.4426950408889634f,
                    lr, lg);
   float l = st.l;
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // With a single slice in the grid the result is written directly.
 #define DECODE_MIN_CHUNK 64
 
-template <int NT>
+template <int NT, bool BIAS>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     uint16_t* __restrict__ out, float* __restrict__ ws_o, float* __restrict__ ws_ml,
     const uint16_t* __restrict__ q,
@@ -148,8 +150,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   for (int dt = 0; dt < NT; ++dt) st.o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   st.m = -INFINITY;
   st.l = 0.f;
+  st.bias = BIAS ? ex.slopes[h] / scale : 0.f;
+  st.pos = n_keys - 1;
   const int hi = n_keys - 1;
-  attend_range<NT, false>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
+  attend_range<NT, false, BIAS>(st, qf, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin,
                    (kb_end + 31) & ~31, first, hi, first, hi, scale * 1.4426950408889634f, lr, lg);
   float l = st.l;
   l = xor32_sum(xor16_sum(l));
@@ -306,8 +310,8 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
                                         int max_keys, void* workspace_f32,
                                         int64_t workspace_floats, int chunk, const void* sinks,
                                         int sinks_dtype, const void* gate, int64_t gate_stride,
-                                        void* stream) {
-  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk};
+                                        const void* slopes_f32, void* stream) {
+  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk, (const float*)slopes_f32};
   HE_REQUIRE(rows >= 0 && H > 0 && KVH > 0 && hd > 0 && max_keys > 0,
              "he_attention_decode_bf16: bad sizes");
   HE_REQUIRE(scale > 0.f, "he_attention_decode_bf16: the score scale must be positive");
@@ -332,12 +336,16 @@ extern "C" int he_attention_decode_bf16(void* out, const void* q, const void* kp
   float* ws_o = (float*)workspace_f32;
   float* ws_ml = ws_o + (int64_t)rows * H * nsplit * hd;
   dim3 grid(nsplit, KVH * head_tiles, rows);
-  ATTN_SWITCH(hd / 16, (attention_decode_kernel<NT><<<grid, 64, 0, s>>>(
-                           (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)q,
-                           (const uint16_t*)kpool, (const uint16_t*)vpool,
-                           (const int32_t*)positions, (const int32_t*)row_seq,
-                           (const int32_t*)seq_slot, (const int32_t*)page_table, max_blocks,
-                           num_pages, H, KVH, head_tiles, window, scale, ex)));
+#define DECODE_ARGS                                                                                    \
+  (uint16_t*)out, ws_o, ws_ml, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
+      (const int32_t*)positions, (const int32_t*)row_seq, (const int32_t*)seq_slot,                    \
+      (const int32_t*)page_table, max_blocks, num_pages, H, KVH, head_tiles, window, scale, ex
+  if (ex.slopes != nullptr) {
+    ATTN_SWITCH(hd / 16, (attention_decode_kernel<NT, true><<<grid, 64, 0, s>>>(DECODE_ARGS)));
+  } else {
+    ATTN_SWITCH(hd / 16, (attention_decode_kernel<NT, false><<<grid, 64, 0, s>>>(DECODE_ARGS)));
+  }
+#undef DECODE_ARGS
   int rc = he_check_launch("he_attention_decode_bf16");
   if (rc || nsplit == 1) return rc;
   attention_merge_kernel<<<dim3(H, rows), 256, 0, s>>>(
@@ -441,8 +449,9 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
                                          int window, float scale, int kernel, int total_rows,
                                          int parts, void* workspace_f32, int64_t workspace_floats,
                                          int chunk, const void* sinks, int sinks_dtype,
-                                         const void* gate, int64_t gate_stride, void* stream) {
-  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk};
+                                         const void* gate, int64_t gate_stride, const void* slopes_f32,
+                                         void* stream) {
+  const AttnExtras ex = {sinks, sinks_dtype, (const uint16_t*)gate, gate_stride, chunk, (const float*)slopes_f32};
   HE_REQUIRE(num_seqs >= 0 && max_q_len >= 0 && H > 0 && KVH > 0 && hd > 0 && total_rows >= 0,
              "he_attention_prefill_bf16: bad sizes");
   HE_REQUIRE(kernel >= 0 && kernel <= 2,
@@ -461,7 +470,9 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  if (kernel == 0) kernel = hd > 128 ? 1 : 2;
+  // the kernel that shares pages through LDS has no distance slopes
+  HE_REQUIRE(slopes_f32 == nullptr || kernel != 2, "he_attention_prefill_bf16: distance slopes are for kernel 1");
+  if (kernel == 0) kernel = (hd > 128 || slopes_f32 != nullptr) ? 1 : 2;
   if (parts < 1) parts = 1;
   HE_REQUIRE(parts == 1 || kernel == 2,
              "he_attention_prefill_bf16: keys in %d parts are for kernel 2 (head sizes up to 128)", parts);
@@ -481,11 +492,15 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
     return he_attention_merge_rows(out, ws_o, ws_ml, total_rows, H, hd, parts, ex, stream);
   }
   dim3 grid((max_q_len + 63) / 64, H, num_seqs);
-  ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT><<<grid, 256, 0, s>>>(
-                           (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool,
-                           (const uint16_t*)vpool, (const int32_t*)cu_seqlens,
-                           (const int32_t*)seq_slot, (const int32_t*)seq_start,
-                           (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window,
-                           scale, ex)));
+#define PREFILL_ARGS                                                                                   \
+  (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,                  \
+      (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,                 \
+      (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale, ex
+  if (ex.slopes != nullptr) {
+    ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT, true><<<grid, 256, 0, s>>>(PREFILL_ARGS)));
+  } else {
+    ATTN_SWITCH(hd / 16, (attention_prefill_kernel<NT, false><<<grid, 256, 0, s>>>(PREFILL_ARGS)));
+  }
+#undef PREFILL_ARGS
   return he_check_launch("he_attention_prefill_bf16");
 }

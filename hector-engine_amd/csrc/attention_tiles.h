@@ -43,6 +43,8 @@ struct AttnState {
   floatx4 o[NT];  // O^T[16*dt + 4*lg + i][q], unnormalised
   float m;        // reference point (near the running maximum) of the query of this lane's column
   float l;        // this lane's share of the running sum
+  float bias;     // BIAS kernels: the raw score of key j gains bias * (j - pos) (a distance slope over the score scale)
+  int pos;        // BIAS kernels: the position of this lane's query
 };
 
 // The K and V^T operands of one step of 32 keys, loaded ahead of their use so that the
@@ -82,7 +84,7 @@ __device__ __forceinline__ void load_frag(KVFrag<NT>& f, const uint16_t* __restr
 // base-2 domain: s2 = (q . k) * scale * log2(e), p = 2^(s2 - m), so the exponential is
 // the bare hardware instruction; m is the reference point of s2 (see HE_SOFTMAX_SLACK). When
 // no query's reference point moves, the rescaling of the accumulators is skipped.
-template <int NT, bool MASK>
+template <int NT, bool MASK, bool BIAS = false>
 __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
                                             const KVFrag<NT>& f, int key_base, int lo, int hi,
                                             float scale_log2, int lg) {
@@ -106,6 +108,7 @@ __device__ __forceinline__ void attend_frag(AttnState<NT>& st, const bf16x8* qf,
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float v = s[t][r];
+      if (BIAS) v = __builtin_fmaf(st.bias, (float)(key_base + 8 * lg + 4 * t + r - st.pos), v);
       if (MASK) {
         const int key = key_base + 8 * lg + 4 * t + r;
         v = (key >= lo && key <= hi) ? v : -INFINITY;
@@ -196,7 +199,7 @@ __device__ __forceinline__ void attend_start(AttendCursor<NT>& c, const uint16_t
 
 // Runs the keys [kb_begin, kb_end) (multiples of 32) of one (sequence, kv head) against the
 // state, one step ahead with its loads and one page ahead with its page-table entry.
-template <int NT, bool UNMASKED_STEPS>
+template <int NT, bool UNMASKED_STEPS, bool BIAS = false>
 __device__ __forceinline__ void attend_walk(AttnState<NT>& st, const bf16x8* qf, AttendCursor<NT>& c,
                                             const int32_t* __restrict__ pt, int max_blocks,
                                             int num_pages, int kb_begin, int kb_end, int lo, int hi,
@@ -215,14 +218,14 @@ __device__ __forceinline__ void attend_walk(AttnState<NT>& st, const bf16x8* qf,
     }
     // keys in [clear_lo, clear_hi] are visible to every query of the tile
     if (UNMASKED_STEPS && kb >= clear_lo && kb + 31 <= clear_hi && c.cur.ok)
-      attend_frag<NT, false>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
+      attend_frag<NT, false, BIAS>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
     else
-      attend_frag<NT, true>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
+      attend_frag<NT, true, BIAS>(st, qf, c.cur, kb, lo, hi, scale_log2, lg);
     c.cur = nxt;
   }
 }
 
-template <int NT, bool UNMASKED_STEPS>
+template <int NT, bool UNMASKED_STEPS, bool BIAS = false>
 __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf,
                                              const uint16_t* __restrict__ kpool,
                                              const uint16_t* __restrict__ vpool,
@@ -233,7 +236,7 @@ __device__ __forceinline__ void attend_range(AttnState<NT>& st, const bf16x8* qf
   if (kb_begin >= kb_end) return;
   AttendCursor<NT> c;
   attend_start<NT>(c, kpool, vpool, pt, max_blocks, num_pages, KVH, kvh, kb_begin, lr, lg);
-  attend_walk<NT, UNMASKED_STEPS>(st, qf, c, pt, max_blocks, num_pages, kb_begin, kb_end, lo, hi,
+  attend_walk<NT, UNMASKED_STEPS, BIAS>(st, qf, c, pt, max_blocks, num_pages, kb_begin, kb_end, lo, hi,
                                   clear_lo, clear_hi, scale_log2, lr, lg);
 }
 

@@ -221,6 +221,7 @@ struct AttnExtras {
   const uint16_t* gate;
   int64_t gate_stride;
   int chunk;
+  const float* slopes;   // [H] or null: the score of key j for the query at p loses slopes[h] * (p - j)
 };
 // attention_mfma.hip: joins attention parts that were all stored (the fused one-token kernel's, the
 // prompt kernel's); row_seq may be null: every row has a sequence

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 27
+#define HE_ABI_VERSION 28
 
 #ifdef __cplusplus
 extern "C" {
@@ -172,7 +172,7 @@ int he_attention_decode_bf16(void* out, const void* q, const void* kpool, const 
                              int H, int KVH, int hd, int window, float scale, int max_keys,
                              void* workspace_f32, int64_t workspace_floats, int chunk,
                              const void* sinks, int sinks_dtype, const void* gate, int64_t gate_stride,
-                             void* stream);
+                             const void* slopes_f32, void* stream);
 int64_t he_attention_decode_workspace_floats(int rows, int H, int KVH, int hd, int max_keys);
 // bf16, one query row per sequence, one launch for bias + rotary + cache write + attention +
 // merge (a second launch joins the parts where few sequences are cut across workgroups).
@@ -213,7 +213,7 @@ int he_attention_prefill_bf16(void* out, const void* q, const void* kpool, const
                               int max_q_len, int H, int KVH, int hd, int window, float scale,
                               int kernel, int total_rows, int parts, void* workspace_f32,
                               int64_t workspace_floats, int chunk, const void* sinks, int sinks_dtype,
-                              const void* gate, int64_t gate_stride, void* stream);
+                              const void* gate, int64_t gate_stride, const void* slopes_f32, void* stream);
 
 // ---- state-space mixer (state_space.hip) ------------------------------------
 // A sequence's row of the state area holds, in fp32, the last K-1 inputs of the convolution [K-1][C] at

@@ -1112,13 +1112,15 @@ def attention_decode_workspace_floats(rows: int, H: int, KVH: int, hd: int, max_
 @_op("attention_decode")
 def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_table, rows: int,
                      H: int, KVH: int, hd: int, window: int, scale: float, max_keys: int,
-                     workspace, *, chunk: int = 0, sinks=None, gate=None) -> None:
-    """chunk, sinks, gate: as attention_plain takes them."""
+                     workspace, *, chunk: int = 0, sinks=None, gate=None, slopes=None) -> None:
+    """chunk, sinks, gate, slopes: as attention_plain takes them."""
     _check_attention(out, q, kpool, vpool, page_table, rows, H, KVH, hd)
     _need(q, "q", torch.bfloat16)
     gate_ptr, gate_stride = _gate_view(gate, q, rows, H)
     if sinks is not None:
         _need(sinks, "sinks", shape=(H,))
+    if slopes is not None:
+        _need(slopes, "slopes", torch.float32, (H,))
     for name, t in (("positions", positions), ("row_seq", row_seq), ("seq_slot", seq_slot)):
         _need(t, name, torch.int32)
     if positions.numel() < rows or row_seq.numel() < rows:
@@ -1130,7 +1132,7 @@ def attention_decode(out, q, kpool, vpool, positions, row_seq, seq_slot, page_ta
         row_seq.data_ptr(), seq_slot.data_ptr(), page_table.data_ptr(), page_table.shape[1],
         kpool.shape[0], rows, H, KVH, hd, window, float(scale), max_keys, workspace.data_ptr(),
         workspace.numel(), int(chunk), _ptr(sinks), dtype_code(sinks.dtype) if sinks is not None else F32,
-        gate_ptr, gate_stride, _stream()))
+        gate_ptr, gate_stride, _ptr(slopes), _stream()))
 
 
 def attention_decode_fused_ok(H: int, KVH: int, hd: int, rotary_dim: int) -> bool:
@@ -1213,17 +1215,20 @@ def attention_prefill_workspace_floats(total_rows: int, H: int, hd: int, parts: 
 def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, page_table,
                       num_seqs: int, max_q_len: int, total_rows: int, H: int, KVH: int, hd: int,
                       window: int, scale: float, kernel: int = 0, parts: int = 1, workspace=None, *,
-                      chunk: int = 0, sinks=None, gate=None) -> None:
+                      chunk: int = 0, sinks=None, gate=None, slopes=None) -> None:
     """kernel: 0 leaves the choice to the library (by head size and prompt length); 1 or 2
     name it: 16 queries a wavefront with operands from global memory, or 32 queries a
     wavefront with the pages shared through LDS (head sizes up to 128). parts > 1 (kernel 2):
     the keys in that many parts side by side, joined by a second launch; the workspace holds
-    attention_prefill_workspace_floats() floats. chunk, sinks, gate: as attention_plain takes them."""
+    attention_prefill_workspace_floats() floats. chunk, sinks, gate, slopes: as attention_plain takes them
+    (with slopes the library's choice is kernel 1 and the keys stay in one part)."""
     _check_attention(out, q, kpool, vpool, page_table, total_rows, H, KVH, hd)
     _need(q, "q", torch.bfloat16)
     gate_ptr, gate_stride = _gate_view(gate, q, total_rows, H)
     if sinks is not None:
         _need(sinks, "sinks", shape=(H,))
+    if slopes is not None:
+        _need(slopes, "slopes", torch.float32, (H,))
     for name, t in (("cu_seqlens", cu_seqlens), ("seq_slot", seq_slot), ("seq_start", seq_start)):
         _need(t, name, torch.int32)
     if cu_seqlens.numel() < num_seqs + 1 or seq_slot.numel() < num_seqs or seq_start.numel() < num_seqs:
@@ -1237,7 +1242,7 @@ def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, pag
         kpool.shape[0], num_seqs, max_q_len, H, KVH, hd, window, float(scale), int(kernel),
         total_rows, int(parts), _ptr(workspace), workspace.numel() if workspace is not None else 0,
         int(chunk), _ptr(sinks), dtype_code(sinks.dtype) if sinks is not None else F32, gate_ptr, gate_stride,
-        _stream()))
+        _ptr(slopes), _stream()))
 
 
 @_op("argmax_rows")

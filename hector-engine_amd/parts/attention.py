@@ -162,8 +162,7 @@ class Attention(Mixer):
         self.o_proj: Linear | None = None
         self._chosen: dict[tuple, routes.Route] = {}      # (all one-token, dtype) -> route, for one version of the table
         self._chosen_version = -1
-        # else the plain kernel (which alone takes the distance slopes)
-        self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0 and not self.slope_span
+        self.fast = mfma and self.pd % 16 == 0 and self.pd <= 256 and self.scale > 0   # else the plain kernel
         # what the fused one-token kernel and the kernels without these options do not take
         self.extras = self.chunk > 0 or self.has_sinks or self.head_gate or self.maps > 1 or self.q_temp is not None \
             or self.out_gate or self.sink_value is not None or bool(self.qk_norm) or self.conv_taps > 0 \
@@ -438,7 +437,8 @@ class Attention(Mixer):
         ws = ctx.alloc((max(floats, 1),), torch.float32)
         ops.attention_decode(out, q, cache.kpool, cache.vpool, ctx.positions, ctx.row_seq,
                              ctx.seq_slot, cache.page_table, rows, H, KVH, hd, self.window,
-                             self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+                             self.scale, ctx.max_keys, ws, chunk=self.chunk, sinks=self.sinks,
+                             gate=gate if self.head_gate else None, slopes=self.slopes)
         return self._project(out, rows, ctx, gate)
 
     def _run_mfma_prompt(self, x, ctx: StepContext, cache: LayerCache):
@@ -452,7 +452,8 @@ class Attention(Mixer):
             most = min(most, self.window + ctx.max_q_len)
         if self.chunk > 0:
             most = min(most, self.chunk + ctx.max_q_len)
-        parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
+        # (the kernel that takes distance slopes walks a query's keys in one part)
+        parts = 1 if self.slopes is not None else ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
         ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
             if parts > 1 else None
         if ctx.padded:
@@ -462,7 +463,8 @@ class Attention(Mixer):
         ops.attention_prefill(out, q, cache.kpool, cache.vpool, ctx.cu_seqlens, ctx.seq_slot,
                               ctx.seq_start, cache.page_table, ctx.num_seqs, ctx.max_q_len,
                               rows, H, KVH, hd, self.window, self.scale, parts=parts, workspace=ws,
-                              chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None)
+                              chunk=self.chunk, sinks=self.sinks, gate=gate if self.head_gate else None,
+                              slopes=self.slopes)
         return self._project(out, rows, ctx, gate)
 
 

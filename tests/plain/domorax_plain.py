@@ -134,6 +134,28 @@ def latent_attention(h, w, pre, m, eps, positions):
     return out.reshape(T, H * e) @ w[pre + "o"].T
 
 
+def head_slopes(H: int):
+    """slope_h = 2^(-8 (h + 1) / H) for head h."""
+    return [2.0 ** (-8.0 * (h + 1) / H) for h in range(H)]
+
+
+def distance_attention(q, k, v, scale, slopes, first_position=0):
+    """q [Tq, H, d] at the positions first_position.., k and v [Tk, G, d] at the positions 0..: causal softmax
+    attention whose score for key j and the query at position i is (q . k) * scale - slope_h * (i - j)."""
+    Tq, H, d = q.shape
+    G = k.shape[1]
+    out = torch.zeros((Tq, H, v.shape[2]), dtype=F64)
+    ahead = torch.arange(k.shape[0], dtype=F64)
+    for head in range(H):
+        g = head // (H // G)
+        for t in range(Tq):
+            i = first_position + t
+            s = (k[:i + 1, g] @ q[t, head]) * scale - slopes[head] * (i - ahead[:i + 1])
+            p = torch.softmax(s, 0)
+            out[t, head] = (p[:, None] * v[:i + 1, g]).sum(0)
+    return out
+
+
 def conv_attention(h, w, pre, m, eps):
     """Grouped-query attention whose q and k pass a short convolution and a per-head norm, whose
     values are the keys as they leave the convolution, and whose scores lose slope_h * distance."""
@@ -144,15 +166,7 @@ def conv_attention(h, w, pre, m, eps):
     v = k
     q = rms(q, eps) * w[pre + "q.norm"]
     k = rms(k, eps) * w[pre + "k.norm"]
-    out = torch.zeros((T, H, d), dtype=F64)
-    ahead = torch.arange(T, dtype=F64)
-    for head in range(H):
-        g = head // (H // G)
-        slope = 2.0 ** (-8.0 * (head + 1) / H)
-        for t in range(T):
-            s = (k[:t + 1, g] @ q[t, head]) * m["scale"] - slope * (t - ahead[:t + 1])
-            p = torch.softmax(s, 0)
-            out[t, head] = (p[:, None] * v[:t + 1, g]).sum(0)
+    out = distance_attention(q, k, v, m["scale"], head_slopes(H))
     return out.reshape(T, H * d) @ w[pre + "o"].T
 
 

@@ -226,7 +226,8 @@ def test_the_mix_over_all_results_so_far(ops):
 def test_the_gate_of_a_shared_expert(ops, dtype):
     tdt = TORCH[dtype]
     rows, D = 9, 50
-    a, b, x, g = (rnd(rows, D, seed=s).to(tdt) for s in (50, 51, 52)) + (rnd(D, seed=53, scale=0.3).to(tdt),)
+    a, b, x = (rnd(rows, D, seed=s).to(tdt) for s in (50, 51, 52))
+    g = rnd(D, seed=53, scale=0.3).to(tdt)
     out = torch.empty(rows, D, dtype=tdt, device="cuda")
     ops.gated_add(out, dev(a), dev(b), dev(x), dev(g), rows)
     want = a.double() + torch.sigmoid(x.double() @ g.double())[:, None] * b.double()
@@ -289,6 +290,59 @@ def test_weights_that_are_the_softmax_over_the_chosen_logits(ops, E, top):
     assert torch.allclose(dense_w[:, :E].cpu().double(), want, atol=1e-6) and float(dense_w[:, E].abs().max()) == 0.0
     assert torch.allclose(weights.cpu().double().sum(-1), torch.ones(rows, dtype=F64), atol=1e-6)
     assert torch.allclose(torch.gather(want, 1, ids.cpu().long()), weights.cpu().double(), atol=1e-6)
+
+
+# ------------------------------------------------------------------ attention with distance slopes
+@pytest.mark.parametrize("kind,dtype", [("plain", "float32"), ("plain", "bfloat16"), ("decode", "bfloat16"), ("prefill", "bfloat16")])
+@pytest.mark.parametrize("H,KVH,hd", [(6, 2, 32), (4, 1, 96), (3, 3, 16), (20, 1, 48), (2, 1, 160)])
+def test_scores_that_fall_with_the_distance(ops, kind, dtype, H, KVH, hd):
+    """Every attention kernel with a slope a head, against the direct sums: prompts, a continuation and single tokens
+    over page edges. One early key of every sequence is made to match the last query, with a score that equals what
+    the slope takes off at that distance: without the slope it would take most of the weight; with it, it is one key
+    among the near ones."""
+    from tests.test_kernels_gpu import fill_cache, paged_setup
+    tdt = TORCH[dtype]
+    lengths, q_lens = ([300, 1, 64, 65, 131], [1, 1, 1, 1, 1]) if kind == "decode" else ([150, 237, 3, 66], [150, 37, 3, 1])
+    slots, table, kpool, vpool = paged_setup(lengths, KVH, hd, tdt, 90)
+    ks = [rnd(n, KVH, hd, seed=100 + i).to(tdt) for i, n in enumerate(lengths)]
+    vs = [rnd(n, KVH, hd, seed=110 + i).to(tdt) for i, n in enumerate(lengths)]
+    qs = [rnd(m, H, hd, seed=120 + i, scale=2.0).to(tdt) for i, m in enumerate(q_lens)]
+    slopes = torch.tensor(P.head_slopes(H), dtype=torch.float32)
+    scale = hd ** -0.5
+    for k, q in zip(ks, qs):
+        n = k.shape[0]
+        if n > 8:
+            first = q[-1, ::H // KVH].float()                        # the last query of each group's first head
+            much = slopes[::H // KVH, None] * (n - 3) / (first.pow(2).sum(-1, keepdim=True) * scale)
+            k[2] = (first * much).to(tdt)                            # key 2 points where that query points
+    fill_cache(table, slots, kpool, vpool, ks, vs)
+    rows = sum(q_lens)
+    q = torch.cat(qs).reshape(rows, H * hd)
+    positions = torch.cat([torch.arange(n - m, n) for n, m in zip(lengths, q_lens)]).int()
+    row_seq = torch.cat([torch.full((m,), i) for i, m in enumerate(q_lens)]).int()
+    cu, starts = cu_of(q_lens), i32([n - m for n, m in zip(lengths, q_lens)])
+    out = torch.full((rows, H * hd), 7.0, dtype=tdt, device="cuda")
+    pools = (dev(kpool), dev(vpool))
+    if kind == "plain":
+        ops.attention_plain(out, dev(q), *pools, dev(positions), dev(row_seq), i32(slots), dev(table), rows, H, KVH, hd, 0,
+                            scale, slopes=dev(slopes))
+    elif kind == "decode":
+        ws = torch.empty(ops.attention_decode_workspace_floats(rows, H, KVH, hd, 4096), device="cuda")
+        ops.attention_decode(out, dev(q), *pools, dev(positions), dev(row_seq), i32(slots), dev(table), rows, H, KVH, hd, 0,
+                             scale, 4096, ws, slopes=dev(slopes))
+    else:
+        ops.attention_prefill(out, dev(q), *pools, cu, i32(slots), starts, dev(table), len(lengths), max(q_lens), rows, H, KVH,
+                              hd, 0, scale, slopes=dev(slopes))
+    r, moved = 0, 0.0
+    for i, (n, m) in enumerate(zip(lengths, q_lens)):
+        want = P.distance_attention(qs[i].double(), ks[i].double(), vs[i].double(), scale, slopes.double().tolist(), n - m)
+        flat = P.distance_attention(qs[i].double(), ks[i].double(), vs[i].double(), scale, [0.0] * H, n - m)
+        got = out[r:r + m].cpu().double().reshape(want.shape)
+        bound = 3e-5 if dtype == "float32" else 2 ** -6          # scores of a hundred, known to 32 bits, under an exponential
+        assert torch.allclose(got, want, rtol=bound, atol=bound)
+        moved = max(moved, (want[-1] - flat[-1]).abs().max().item())
+        r += m
+    assert moved > 0.3          # the slope decides here
 
 
 # ------------------------------------------------------------------ whole models through the engine
