@@ -4,7 +4,7 @@ token ids) on one MI355X, with prefill and roofline figures on the same line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b|32b|72b]
                     [--context C] [--prompt P]
-    python bench.py --design volonex | penasun | butolorn      (another measurement: see below)
+    python bench.py --design volonex | penasun | butolorn | domorax      (another measurement: see below)
 
 The default is the 7B shape; --shape runs the same measurement at the layer sizes of
 Qwen2.5-32B (context 8192, prompts of 512 to 2048 tokens, batches 1 / 8 / 64) or
@@ -28,8 +28,8 @@ the machine runs every kernel of the one-token step 4 to 6 % slower than afterwa
 leaves its first run and its thermal-low samples out: OPTIMIZATION_NOTES.md:114-117); `repeats` holds
 every timed run, the earlier ones still show it.
 
---design volonex (or penasun; butolorn is measured beside Penasun, the other design whose layers carry a state
-of fixed size) leaves the run above aside and measures that design beside Qwen2 at equal layer
+--design volonex (or penasun; butolorn and domorax are measured beside Penasun, the other design whose layers carry
+a state of fixed size) leaves the run above aside and measures that design beside Qwen2 at equal layer
 sizes (random weights, bf16, four layers of each of a few sizes that resemble real models' layers): prompt
 tokens a second for one prompt of 2,048 tokens, decoded tokens a second at batch 8 and batch 1 behind such
 prompts, and, from a second pass with an event pair around every launch, the mean time of each kind of
@@ -159,6 +159,31 @@ def butolorn_configs(sz):
     return penasun, config_from_dict(butolorn)
 
 
+def domorax_configs(sz):
+    """(Penasun configuration, Domorax configuration) of one set of layer sizes. Penasun is the design beside it: both
+    have layers that carry a state of fixed size per sequence behind a short convolution, attention layers, and a
+    routed feed-forward. The Domorax layers are a gated delta rule (heads of the Qwen2 layer's key and value widths), an
+    attention through latents (as many heads; 64 rotated dims, a latent of 192, so that the one cached key is 256
+    wide; a window of 1,024), a delta rule again with a dense feed-forward of the Qwen2 layer's width, and a convolved
+    attention with distance slopes whose values are its keys; the other layers route 4 of 16 experts, each a
+    quarter of the Qwen2 feed-forward wide, beside a shared expert of that width."""
+    from hector_engine_amd.registry import config_from_dict
+    _, penasun = penasun_configs(sz)
+    delta = dict(type="delta", mixer=dict(heads=sz["heads"], kv_heads=sz["kv_heads"], dim=sz["dim"], vdim=sz["vdim"], conv=4))
+    latent = dict(type="latent_attention", mixer=dict(
+        heads=sz["heads"], dim=sz["dim"], rot_dim=64, vdim=sz["vdim"], kv_rank=192, q_rank=sz["width"] // 2,
+        scale=(sz["dim"] + 64) ** -0.5, mask=dict(size=1024),
+        rot=dict(base=10000.0, dims=64, scaling=dict(factor=4.0, original=1024, fast=32.0, slow=1.0))))
+    wide = max(sz["dim"], sz["vdim"])
+    attention = dict(type="attention", mixer=dict(heads=sz["heads"], kv_heads=sz["kv_heads"], dim=wide, vdim=wide, conv=4,
+                                                  scale=wide ** -0.5))
+    moe = dict(kind="moe", expert=dict(ff=sz["ff"] // 4), router=dict(experts=16, top=4), shared=dict(ff=sz["ff"] // 4))
+    layers = [dict(delta, mlp=moe), dict(latent, mlp=moe), dict(delta, mlp=dict(kind="dense", ff=sz["ff"])), dict(attention, mlp=moe)]
+    domorax = dict(architecture="Domorax", vocab=DESIGN_VOCAB, width=sz["width"], residual_mult=0.5,
+                   norm=dict(eps=1e-6, groups=4), layers=layers)
+    return penasun, config_from_dict(domorax)
+
+
 def compare_designs(args) -> int:
     import torch
     import hector_engine_amd as he
@@ -237,12 +262,13 @@ def compare_designs(args) -> int:
         return out
 
     result = {}
-    beside = "penasun" if args.design == "butolorn" else "qwen2"
+    beside = "penasun" if args.design in ("butolorn", "domorax") else "qwen2"
     chosen = [n for n in DESIGN_SIZES if not args.design_sizes or n in args.design_sizes.split(",")]
     for name in chosen:
         sz = DESIGN_SIZES[name]
         result[name] = {"sizes": sz}
-        configs = {"volonex": design_configs, "penasun": penasun_configs, "butolorn": butolorn_configs}[args.design](sz)
+        configs = {"volonex": design_configs, "penasun": penasun_configs, "butolorn": butolorn_configs,
+                   "domorax": domorax_configs}[args.design](sz)
         for design, config in zip((beside, args.design), configs):
             progress(f"{name} {design}")
             result[name][design] = measure(config, False)
@@ -283,8 +309,8 @@ def main() -> int:
     ap.add_argument("--no-tune", action="store_true",
                     help="leave the library's default kernels for the tall matrix products")
     ap.add_argument("--design-sizes", default="", help=f"with --design: only these of {', '.join(DESIGN_SIZES)}")
-    ap.add_argument("--design", choices=["volonex", "penasun", "butolorn"], default=None,
-                    help="instead of the run above: this design beside Qwen2 (butolorn: beside Penasun) at equal layer sizes, prompt and "
+    ap.add_argument("--design", choices=["volonex", "penasun", "butolorn", "domorax"], default=None,
+                    help="instead of the run above: this design beside Qwen2 (butolorn, domorax: beside Penasun) at equal layer sizes, prompt and "
                          "one-token steps, throughput and mean time per kind of kernel")
     args = ap.parse_args()
     if args.design:

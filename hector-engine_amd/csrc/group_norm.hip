@@ -88,7 +88,7 @@ extern "C" int he_add_group_normed(void* resid_f32, const void* delta, int delta
 // out[r, i] = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e over the W values z of row r, with
 // rms(x) = sqrt(mean(x^2) + eps) and the four numbers (a, b, c, e) in `numbers`. out may be x itself.
 template <typename T>
-__global__ __launch_bounds__(256) void polynorm_kernel(T* out, const T* x,
+__global__ __launch_bounds__(1024) void polynorm_kernel(T* out, const T* x,
                                                         const void* __restrict__ numbers, int n_dtype, int W, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
@@ -121,7 +121,8 @@ extern "C" int he_polynorm(void* out, const void* x, const void* numbers, int n_
   HE_REQUIRE(rows >= 0 && W > 0, "he_polynorm: bad sizes rows=%d W=%d", rows, W);
   HE_REQUIRE((dtype == HE_BF16 || dtype == HE_F32) && (n_dtype == HE_BF16 || n_dtype == HE_F32), "he_polynorm: unknown dtype");
   if (rows == 0) return 0;
-  const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+  // few rows: a row's elements over as many threads as a workgroup has; many rows fill the chip anyway
+  const int threads = rows <= 64 && W >= 8192 ? 1024 : rows <= 64 && W >= 4096 ? 512 : W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
   hipStream_t s = (hipStream_t)stream;
   if (dtype == HE_BF16)
     polynorm_kernel<bf16_t><<<rows, threads, 0, s>>>((bf16_t*)out, (const bf16_t*)x, numbers, n_dtype, W, eps);

@@ -6,7 +6,7 @@
 #pragma once
 #include <stdint.h>
 
-#define HE_ABI_VERSION 28
+#define HE_ABI_VERSION 29
 
 #ifdef __cplusplus
 extern "C" {
@@ -326,11 +326,14 @@ int he_scaled_sum(void* out, const void* a, const void* b, int64_t n, float sa, 
 // q, k to unit length (q times q_scale), beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)); S <- g S;
 // u = beta (v - S^T k); S <- S + k u^T; y = S^T q. S (fp32, he_delta_state_floats floats) lives at byte state_offset of the
 // sequence's row of the state area and is carried on.
+// workspace_f32: he_delta_workspace_floats floats (16-byte aligned) for what a first launch prepares row by row.
 int64_t he_delta_state_floats(int H, int d, int e);
+int64_t he_delta_workspace_floats(int rows, int H, int G, int d);
 int he_delta_scan(void* y_f32, const void* q, const void* k, const void* v, int64_t in_stride, const void* ba_f32,
                   const void* a_log, const void* dt_bias, int w_dtype, void* state, int64_t state_stride,
                   int64_t state_offset, const void* cu_seqlens, const void* seq_slot, int rows, int num_seqs, int H, int G,
-                  int d, int e, float q_scale, float unit_eps, int dtype, void* stream);
+                  int d, int e, float q_scale, float unit_eps, void* workspace_f32, int64_t workspace_floats, int dtype,
+                  void* stream);
 
 // ---- norms over parts of a row (group_norm.hip) --------------------------------------------------------
 // resid += delta_scale * gn(delta) with gn the RMS norm in `groups` equal consecutive parts times weight (delta null:

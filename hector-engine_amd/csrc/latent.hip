@@ -10,21 +10,26 @@
 
 #define HP_ROWS 8
 #define HP_KCHUNK 256
-// out[r, h, n] = sum_k x[r, h, k] * w[h, k, n], k ascending in one chain of multiply-adds, in fp32.
-// x at x_row / x_head element strides, out likewise; w [H][K][N]. A workgroup takes HP_ROWS rows of one head
-// and 64 to 256 neighbouring n; the rows' x values are staged in LDS a chunk of K at a time.
+// out[r, h, n] = sum_k x[r, h, k] * w[h, k, n] in fp32: k in chunks of HP_KCHUNK; inside a chunk each of the
+// workgroup's four wavefronts takes a quarter of the k (a chain of multiply-adds in ascending k, eight weight loads
+// in flight), the four sums meet in wavefront order, and the chunks' sums are added in chunk order: one order a
+// row whatever else the step holds. x at x_row / x_head element strides, out likewise; w [H][K][N]. A workgroup
+// takes HP_ROWS rows of one head and 64 neighbouring n; the rows' x values are staged in LDS a chunk at a time.
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void head_product_kernel(T* __restrict__ out, int64_t o_row, int64_t o_head,
                                                            const T* __restrict__ x, int64_t x_row, int64_t x_head,
                                                            const TW* __restrict__ w, int rows, int K, int N) {
   __shared__ float xs[HP_ROWS][HP_KCHUNK];
+  __shared__ float part[4][HP_ROWS][64];
   const int h = blockIdx.y;
   const int64_t r0 = (int64_t)blockIdx.z * HP_ROWS;
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + lane;
+  const int nc = min(n, N - 1);            // a lane beyond N reads the last column and stores nothing
   const TW* wh = w + (int64_t)h * K * N;
-  float acc[HP_ROWS];
+  float total[HP_ROWS];
 #pragma unroll
-  for (int r = 0; r < HP_ROWS; ++r) acc[r] = 0.f;
+  for (int r = 0; r < HP_ROWS; ++r) total[r] = 0.f;
   for (int k0 = 0; k0 < K; k0 += HP_KCHUNK) {
     const int kc = min(HP_KCHUNK, K - k0);
     __syncthreads();
@@ -33,18 +38,92 @@ __global__ __launch_bounds__(256) void head_product_kernel(T* __restrict__ out, 
       xs[r][k] = r0 + r < rows ? to_float(x[(r0 + r) * x_row + h * x_head + k0 + k]) : 0.f;
     }
     __syncthreads();
-    if (n < N) {
-      for (int k = 0; k < kc; ++k) {
-        const float wv = to_float(wh[(int64_t)(k0 + k) * N + n]);
+    const int per = (kc + 3) / 4;
+    const int ka = wave * per, kb = min(kc, ka + per);
+    float acc[HP_ROWS];
 #pragma unroll
-        for (int r = 0; r < HP_ROWS; ++r) acc[r] = fmaf(xs[r][k], wv, acc[r]);
+    for (int r = 0; r < HP_ROWS; ++r) acc[r] = 0.f;
+    for (int k = ka; k < kb; k += 8) {
+      float wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(int64_t)(k0 + min(k + u, kb - 1)) * N + nc]);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (k + u < kb) {
+#pragma unroll
+          for (int r = 0; r < HP_ROWS; ++r) acc[r] = fmaf(xs[r][k + u], wv[u], acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < HP_ROWS; ++r) part[wave][r][lane] = acc[r];
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int r = 0; r < HP_ROWS; ++r)
+        total[r] += ((part[0][r][lane] + part[1][r][lane]) + part[2][r][lane]) + part[3][r][lane];
+    }
+  }
+  if (wave != 0 || n >= N) return;
+#pragma unroll
+  for (int r = 0; r < HP_ROWS; ++r)
+    if (r0 + r < rows) out[(r0 + r) * o_row + h * o_head + n] = from_float<T>(total[r]);
+}
+
+// The same sums in the same order for a step of many rows: a workgroup takes 4 x HP_ROWS rows (a wavefront each
+// HP_ROWS of them) of one head and 64 neighbouring n; a lane forms the four quarter sums of a chunk one after the
+// other and adds them as the kernel above does, so a row has the same bits whichever kernel ran it.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void head_product_rows_kernel(T* __restrict__ out, int64_t o_row, int64_t o_head,
+                                                                const T* __restrict__ x, int64_t x_row, int64_t x_head,
+                                                                const TW* __restrict__ w, int rows, int K, int N) {
+  __shared__ float xs[4 * HP_ROWS][HP_KCHUNK];
+  const int h = blockIdx.y;
+  const int64_t b0 = (int64_t)blockIdx.z * 4 * HP_ROWS;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + lane;
+  const int nc = min(n, N - 1);
+  const TW* wh = w + (int64_t)h * K * N;
+  float total[HP_ROWS];
+#pragma unroll
+  for (int r = 0; r < HP_ROWS; ++r) total[r] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += HP_KCHUNK) {
+    const int kc = min(HP_KCHUNK, K - k0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < 4 * HP_ROWS * kc; i += blockDim.x) {
+      const int r = i / kc, k = i % kc;
+      xs[r][k] = b0 + r < rows ? to_float(x[(b0 + r) * x_row + h * x_head + k0 + k]) : 0.f;
+    }
+    __syncthreads();
+    const int per = (kc + 3) / 4;
+    float quarter[4][HP_ROWS];
+#pragma unroll
+    for (int part = 0; part < 4; ++part) {
+      const int ka = part * per, kb = min(kc, ka + per);
+#pragma unroll
+      for (int r = 0; r < HP_ROWS; ++r) quarter[part][r] = 0.f;
+      for (int k = ka; k < kb; k += 8) {
+        float wv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(int64_t)(k0 + min(k + u, kb - 1)) * N + nc]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (k + u < kb) {
+#pragma unroll
+            for (int r = 0; r < HP_ROWS; ++r)
+              quarter[part][r] = fmaf(xs[wave * HP_ROWS + r][k + u], wv[u], quarter[part][r]);
+          }
       }
     }
+#pragma unroll
+    for (int r = 0; r < HP_ROWS; ++r)
+      total[r] += ((quarter[0][r] + quarter[1][r]) + quarter[2][r]) + quarter[3][r];
   }
   if (n >= N) return;
 #pragma unroll
-  for (int r = 0; r < HP_ROWS; ++r)
-    if (r0 + r < rows) out[(r0 + r) * o_row + h * o_head + n] = from_float<T>(acc[r]);
+  for (int r = 0; r < HP_ROWS; ++r) {
+    const int64_t row = b0 + wave * HP_ROWS + r;
+    if (row < rows) out[row * o_row + h * o_head + n] = from_float<T>(total[r]);
+  }
 }
 
 extern "C" int he_head_product(void* out, int64_t o_row, int64_t o_head, const void* x, int64_t x_row, int64_t x_head,
@@ -52,17 +131,27 @@ extern "C" int he_head_product(void* out, int64_t o_row, int64_t o_head, const v
   HE_REQUIRE(rows >= 0 && H > 0 && K > 0 && N > 0 && H <= 65535, "he_head_product: bad sizes H=%d K=%d N=%d", H, K, N);
   HE_REQUIRE((dtype == HE_BF16 || dtype == HE_F32) && (w_dtype == HE_BF16 || w_dtype == HE_F32), "he_head_product: unknown dtype");
   if (rows == 0) return 0;
-  const int threads = N >= 256 ? 256 : (N >= 128 ? 128 : 64);
-  const dim3 grid((N + threads - 1) / threads, H, (rows + HP_ROWS - 1) / HP_ROWS);
+  const int threads = 256;
+  const bool many = rows > 4 * HP_ROWS;      // a step of many rows: a wavefront takes whole rows, not a quarter of the k
+  const int per_group = many ? 4 * HP_ROWS : HP_ROWS;
+  const dim3 grid((N + 63) / 64, H, (rows + per_group - 1) / per_group);
   HE_REQUIRE(grid.z <= 65535, "he_head_product: %d rows are too many for one launch", rows);
   hipStream_t s = (hipStream_t)stream;
-#define HP_LAUNCH(T, TW)                                                                                             \
-  head_product_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head, (const TW*)w, \
-                                                      rows, K, N)
-  if (dtype == HE_BF16) {
-    if (w_dtype == HE_BF16) HP_LAUNCH(bf16_t, bf16_t); else HP_LAUNCH(bf16_t, float);
+#define HP_LAUNCH(T, TW)                                                                                              \
+  if (many)                                                                                                           \
+    head_product_rows_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head,      \
+                                                             (const TW*)w, rows, K, N);                               \
+  else                                                                                                                \
+    head_product_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head,           \
+                                                        (const TW*)w, rows, K, N)
+  if (dtype == HE_BF16 && w_dtype == HE_BF16) {
+    HP_LAUNCH(bf16_t, bf16_t);
+  } else if (dtype == HE_BF16) {
+    HP_LAUNCH(bf16_t, float);
+  } else if (w_dtype == HE_BF16) {
+    HP_LAUNCH(float, bf16_t);
   } else {
-    if (w_dtype == HE_BF16) HP_LAUNCH(float, bf16_t); else HP_LAUNCH(float, float);
+    HP_LAUNCH(float, float);
   }
 #undef HP_LAUNCH
   return he_check_launch("he_head_product");

@@ -16,7 +16,7 @@ _lib = None
 
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 
-EXPECTED_ABI = 28
+EXPECTED_ABI = 29
 
 c_int, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 
@@ -77,7 +77,8 @@ _SIGNATURES = {
                         c_int, c_int, c_int, c_f32, c_int, c_ptr],
     "he_delta_state_floats": [c_int, c_int, c_int],
     "he_delta_scan": [c_ptr, c_ptr, c_ptr, c_ptr, c_i64, c_ptr, c_ptr, c_ptr, c_int, c_ptr, c_i64, c_i64, c_ptr, c_ptr,
-                      c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_int, c_ptr],
+                      c_int, c_int, c_int, c_int, c_int, c_int, c_f32, c_f32, c_ptr, c_i64, c_int, c_ptr],
+    "he_delta_workspace_floats": [c_int, c_int, c_int, c_int],
     "he_add_group_normed": [c_ptr, c_ptr, c_int, c_ptr, c_int, c_int, c_f32, c_f32, c_ptr, c_int, c_ptr, c_int, c_f32,
                             c_int, c_int, c_ptr],
     "he_polynorm": [c_ptr, c_ptr, c_ptr, c_int, c_int, c_int, c_f32, c_int, c_ptr],
@@ -123,6 +124,7 @@ _RESTYPES = {
     "he_ssm_state_floats": c_i64,
     "he_mlstm_state_floats": c_i64,
     "he_delta_state_floats": c_i64,
+    "he_delta_workspace_floats": c_i64,
     "he_gemm_plain_workspace_floats": c_i64,
     "he_attention_decode_workspace_floats": c_i64,
     "he_attention_decode_fused_workspace_floats": c_i64,

@@ -660,15 +660,23 @@ def delta_state_floats(H: int, d: int, e: int) -> int:
     return int(_lib.load().he_delta_state_floats(H, d, e))
 
 
+def delta_workspace_floats(rows: int, H: int, G: int, d: int) -> int:
+    """Floats of the rows delta_scan prepares before it walks them (unit vectors, gates)."""
+    return int(_lib.load().he_delta_workspace_floats(rows, H, G, d))
+
+
 @_op("delta_scan")
 def delta_scan(y, q, k, v, ba, a_log, dt_bias, state, state_offset: int, cu_seqlens, seq_slot, rows: int,
-               num_seqs: int, H: int, G: int, d: int, e: int, q_scale: float, unit_eps: float) -> None:
+               num_seqs: int, H: int, G: int, d: int, e: int, q_scale: float, unit_eps: float, workspace=None) -> None:
     """y (fp32 [rows, H e]) = the gated delta rule over q, k [rows, G d] and v [rows, H e] (views of rows of one
     buffer, unit stride along the columns), ba (fp32 [rows, 2 H]: write strengths, then decay inputs, both before
     their sigmoid / softplus) and per head a_log, dt_bias; the state [H][e][d'] lives at byte state_offset of a
-    sequence's row of `state` and is carried on."""
+    sequence's row of `state` and is carried on. workspace: fp32, delta_workspace_floats elements or more (None: made here)."""
     _need(y, "y", torch.float32, (None, H * e))
     _need(ba, "ba", torch.float32, (None, 2 * H))
+    if workspace is None:
+        workspace = torch.empty(max(4, delta_workspace_floats(rows, H, G, d)), dtype=torch.float32, device=y.device)
+    _need(workspace, "workspace", torch.float32)
     stride = q.stride(0)
     for name, t, width in (("q", q, G * d), ("k", k, G * d), ("v", v, H * e)):
         if not t.is_cuda or t.dtype != q.dtype or t.dim() != 2 or t.shape[1] != width or t.stride(1) != 1 \
@@ -689,7 +697,8 @@ def delta_scan(y, q, k, v, ba, a_log, dt_bias, state, state_offset: int, cu_seql
     _lib.check(L.he_delta_scan(y.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), stride, ba.data_ptr(),
                                a_log.data_ptr(), dt_bias.data_ptr(), dtype_code(a_log.dtype), state.data_ptr(),
                                state.stride(0), state_offset, cu_seqlens.data_ptr(), seq_slot.data_ptr(), rows, num_seqs,
-                               H, G, d, e, float(q_scale), float(unit_eps), dtype_code(q.dtype), _stream()))
+                               H, G, d, e, float(q_scale), float(unit_eps), workspace.data_ptr(), workspace.numel(),
+                               dtype_code(q.dtype), _stream()))
 
 
 @_op("add_group_normed")

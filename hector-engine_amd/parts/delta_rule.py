@@ -38,14 +38,11 @@ register_init("delta_dt_bias", lambda init: (-1.0, 0.5))
 def state_floats(H: int, d: int, e: int) -> int:
     """Floats of the heads' matrices as the scan kernel keeps them (the rule of csrc/delta_rule.hip, kept here
     so that the cache can be sized where no kernel library is loaded): a value dim's column is held by a power
-    of two of lanes with 8 to 32 key dims each, in steps of 8."""
-    g = 1
-    while g <= 64:
-        per = (-(-d // g) + 7) // 8 * 8
-        if per <= 32:
-            return H * e * g * per
-        g *= 2
-    raise ValueError(f"gated_delta: key width {d} above 2048")
+    of two of lanes with 8 to 32 key dims each, in steps of 8, the fewest dims in all."""
+    padded = [g * per for g in (1, 2, 4, 8, 16, 32, 64) for per in [(-(-d // g) + 7) // 8 * 8] if per <= 32]
+    if not padded:
+        raise ValueError(f"gated_delta: key width {d} above 2048")
+    return H * e * min(padded)
 
 
 @register_part("mixer", "gated_delta")
@@ -122,9 +119,10 @@ class GatedDeltaRule(Mixer):
         y = ctx.alloc((rows, H * e), torch.float32)
         if ctx.padded:
             y.zero_()           # the scan writes the rows of sequences only
+        ws = ctx.alloc((max(4, ops.delta_workspace_floats(rows, H, G, d)),), torch.float32)
         ops.delta_scan(y, qkv[:, :G * d], qkv[:, G * d:2 * G * d], qkv[:, 2 * G * d:], ba, self.a_log, self.dt_bias,
                        cache.state, self._conv_bytes(), ctx.cu_seqlens, ctx.seq_slot, rows, ctx.num_seqs, H, G, d, e,
-                       self.q_scale, self.unit_eps)
+                       self.q_scale, self.unit_eps, workspace=ws)
         out = ctx.alloc((rows, H * e))
         ops.gated_group_norm(out, y, proj[:, C:], self.norm, rows, H, self.eps, gate_after="silu")
         return self.o_proj(out, rows, ctx, sink=ctx.take_sink())
