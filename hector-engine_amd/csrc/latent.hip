@@ -43,20 +43,16 @@ __global__ __launch_bounds__(256) void head_product_kernel(T* __restrict__ out, 
     float acc[HP_ROWS];
 #pragma unroll
     for (int r = 0; r < HP_ROWS; ++r) acc[r] = 0.f;
-    int k = ka;
-    for (; k + 8 <= kb; k += 8) {          // whole groups of eight k: eight weight loads in flight, no checks
+    for (int k = ka; k < kb; k += 8) {
       float wv[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(int64_t)(k0 + k + u) * N + nc]);
+      for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(int64_t)(k0 + min(k + u, kb - 1)) * N + nc]);
 #pragma unroll
       for (int u = 0; u < 8; ++u)
+        if (k + u < kb) {
 #pragma unroll
-        for (int r = 0; r < HP_ROWS; ++r) acc[r] = fmaf(xs[r][k + u], wv[u], acc[r]);
-    }
-    for (; k < kb; ++k) {
-      const float wv = to_float(wh[(int64_t)(k0 + k) * N + nc]);
-#pragma unroll
-      for (int r = 0; r < HP_ROWS; ++r) acc[r] = fmaf(xs[r][k], wv, acc[r]);
+          for (int r = 0; r < HP_ROWS; ++r) acc[r] = fmaf(xs[r][k + u], wv[u], acc[r]);
+        }
     }
 #pragma unroll
     for (int r = 0; r < HP_ROWS; ++r) part[wave][r][lane] = acc[r];
@@ -105,18 +101,8 @@ __global__ __launch_bounds__(256) void head_product_rows_kernel(T* __restrict__ 
       const int ka = part * per, kb = min(kc, ka + per);
 #pragma unroll
       for (int r = 0; r < HP_ROWS; ++r) quarter[part][r] = 0.f;
-      int k = ka;
-      for (; k + 8 <= kb; k += 8) {
-        float wv[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) wv[u] = to_float(wh[(int64_t)(k0 + k + u) * N + nc]);
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-#pragma unroll
-          for (int r = 0; r < HP_ROWS; ++r)
-            quarter[part][r] = fmaf(xs[wave * HP_ROWS + r][k + u], wv[u], quarter[part][r]);
-      }
-      for (; k < kb; ++k) {
+      // a plain loop: with many rows the other wavefronts hide a load's way (eight loads at a time were slower here)
+      for (int k = ka; k < kb; ++k) {
         const float wv = to_float(wh[(int64_t)(k0 + k) * N + nc]);
 #pragma unroll
         for (int r = 0; r < HP_ROWS; ++r) quarter[part][r] = fmaf(xs[wave * HP_ROWS + r][k], wv, quarter[part][r]);
