@@ -470,9 +470,7 @@ extern "C" int he_attention_prefill_bf16(void* out, const void* q, const void* k
              "he_attention_prefill_bf16: buffers must be 16-byte aligned");
   if (num_seqs == 0 || max_q_len == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  // the kernel that shares pages through LDS has no distance slopes
-  HE_REQUIRE(slopes_f32 == nullptr || kernel != 2, "he_attention_prefill_bf16: distance slopes are for kernel 1");
-  if (kernel == 0) kernel = (hd > 128 || slopes_f32 != nullptr) ? 1 : 2;
+  if (kernel == 0) kernel = hd > 128 ? 1 : 2;
   if (parts < 1) parts = 1;
   HE_REQUIRE(parts == 1 || kernel == 2,
              "he_attention_prefill_bf16: keys in %d parts are for kernel 2 (head sizes up to 128)", parts);

@@ -74,6 +74,7 @@ struct WideTile {
   floatx16 o[Pw<NT>::DT];    // O^T[32dt + 8a + 4g + r][query], i = 4a + r, unnormalised
   float m, l;                // reference point of the lane's query; this lane's share of the sum
   int lo, hi;                // keys the lane's query sees
+  float bias;                // BIAS kernels: the raw score of key j gains bias * (j - hi) (a distance slope over the scale)
 };
 
 // position of score i of a lane of half g inside its step of 32 keys
@@ -135,12 +136,26 @@ __device__ __forceinline__ void pw_epoch_end() {
   __syncthreads();
 }
 
-template <int NT>
-__device__ __forceinline__ floatx16 pw_scores(const bf16x8 (&qf)[NT], const uint4* k_lds, int kl, int hh) {
-  constexpr int KS = Pw<NT>::KS;
+// What the score product of the step from key_base on starts from: zeros, or, with a distance slope, the slope's
+// share of every score, bias * (key - pos): the product adds q . k on top of it, so the softmax sees the sum.
+template <bool BIAS>
+__device__ __forceinline__ floatx16 pw_score_start(float bias, int pos, int key_base, int g) {
   floatx16 s;
+  if (BIAS) {
+    const float base = bias * (float)(key_base + 8 * g - pos);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int i = 0; i < 16; ++i) s[i] = __builtin_fmaf(bias, (float)pw_key_of(i, 0), base);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+  }
+  return s;
+}
+
+template <int NT>
+__device__ __forceinline__ floatx16 pw_scores(const bf16x8 (&qf)[NT], const uint4* k_lds, int kl, int hh,
+                                              floatx16 s) {
+  constexpr int KS = Pw<NT>::KS;
 #pragma unroll
   for (int kk = 0; kk < NT; ++kk) {
     const bf16x8 kf = __builtin_bit_cast(bf16x8, k_lds[kl + hh * 2 * KS * 64 + (kk >> 1) * 64 + (kk & 1) * 32]);
@@ -218,7 +233,7 @@ __device__ __forceinline__ void pw_rescale(WideTile<NT>& t, float alpha) {
 
 // One epoch with masks and range checks: steps hsA..hsB are the tile's. s_pend / p_pend as
 // described at the top. k_lds: page j, v_lds: page j - 1.
-template <int NT>
+template <int NT, bool BIAS>
 __device__ __forceinline__ void pw_plain_epoch(WideTile<NT>& t, floatx16& s_pend, bf16x8 (&p_pend)[2], int j,
                                                int hsA, int hsB, const uint4* k_lds, const uint4* v_lds,
                                                int kl, int vl, int vl_last, int g, float scale_log2) {
@@ -231,10 +246,10 @@ __device__ __forceinline__ void pw_plain_epoch(WideTile<NT>& t, floatx16& s_pend
     pw_values<NT>(t.o, v_lds, vl, vl_last, 1, p);
   }
   if (h2 >= hsA && h2 <= hsB) {
-    const floatx16 s = pw_scores<NT>(t.qf, k_lds, kl, 0);
+    const floatx16 s = pw_scores<NT>(t.qf, k_lds, kl, 0, pw_score_start<BIAS>(t.bias, t.hi, 32 * h2, g));
     if (pw_softmax<NT>(t, s, 32 * h2, g, scale_log2, p_pend, alpha)) pw_rescale<NT>(t, alpha);
   }
-  if (h3 >= hsA && h3 <= hsB) s_pend = pw_scores<NT>(t.qf, k_lds, kl, 1);
+  if (h3 >= hsA && h3 <= hsB) s_pend = pw_scores<NT>(t.qf, k_lds, kl, 1, pw_score_start<BIAS>(t.bias, t.hi, 32 * h3, g));
 }
 
 // One step of the loop without masks: the softmax of the scores in s_pend (step h) beside
@@ -244,11 +259,11 @@ __device__ __forceinline__ void pw_plain_epoch(WideTile<NT>& t, floatx16& s_pend
 // ahead of its product would stall the wavefront for the LDS latency every time); with STAGE
 // the loads of the next pages are issued then, while the first operand is on its way; then
 // the products, each with its piece of the softmax behind it.
-template <int NT, bool STAGE>
+template <int NT, bool STAGE, bool BIAS>
 __device__ __forceinline__ void pw_fast_step(WideTile<NT>& t, floatx16& s_pend, bf16x8 (&p_pend)[2],
                                              const uint4* k_lds, const uint4* v_lds, int kl, int vl,
                                              int vl_last, int hh, int g, float scale_log2,
-                                             PwNext& next, int wave) {
+                                             PwNext& next, int wave, int next_key_base) {
   constexpr int KS = Pw<NT>::KS, DT = Pw<NT>::DT;
   bf16x8 vf[DT][2], kf[NT];
 #pragma unroll
@@ -278,9 +293,7 @@ __device__ __forceinline__ void pw_fast_step(WideTile<NT>& t, floatx16& s_pend, 
   // each, four that round two pairs and add them up; product n of P gets the pieces
   // ceil(16 n / P) .. ceil(16 (n + 1) / P) - 1.
   constexpr int P = NT + 2 * DT;
-  floatx16 s_next;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) s_next[i] = 0.f;
+  floatx16 s_next = pw_score_start<BIAS>(t.bias, t.hi, next_key_base, g);   // the scores of the step at next_key_base
   float mx = -INFINITY, m_new = t.m, sum = 0.f;
   bool moved = false;
   float e[16];
@@ -335,7 +348,7 @@ __device__ __forceinline__ void pw_fast_step(WideTile<NT>& t, floatx16& s_pend, 
   s_pend = s_next;
 }
 
-template <int NT>
+template <int NT, bool BIAS>
 __global__ __launch_bounds__(64 * PW_WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 attention_prefill_wide_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q,
@@ -419,6 +432,7 @@ attention_prefill_wide_kernel(
   t.lo = attn_first(t.hi, window, ex.chunk);
   t.m = -INFINITY;
   t.l = 0.f;
+  t.bias = BIAS ? ex.slopes[h] / scale : 0.f;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -459,7 +473,7 @@ attention_prefill_wide_kernel(
   for (; j < jF0; ++j) {
     if (j + 1 <= pbB) pw_stage<Pw<NT>::K_CHUNKS>(k_base + ((j + 1) & 1) * KP * 16, pw_page(kp, pt[j + 1], num_pages, k_stride, lane), wave);
     if (j <= pbB) pw_stage<Pw<NT>::V_CHUNKS>(v_base + (j & 1) * VP * 16, pw_page(vp, pt[j], num_pages, v_stride, lane), wave);
-    pw_plain_epoch<NT>(t, s_pend, p_pend, j, hsA, hsB, k_lds + (j & 1) * KP, v_lds + ((j - 1) & 1) * VP, kl, vl,
+    pw_plain_epoch<NT, BIAS>(t, s_pend, p_pend, j, hsA, hsB, k_lds + (j & 1) * KP, v_lds + ((j - 1) & 1) * VP, kl, vl,
                        vl_last, g, scale_log2);
     pw_epoch_end();
   }
@@ -480,8 +494,8 @@ attention_prefill_wide_kernel(
     next.v_src = pw_page(vp, page_v, num_pages, v_stride, lane);   // j <= pbB: the tile's own keys lie beyond step 2j
     const uint4* kb = k_lds + (j & 1) * KP;
     const uint4* vb = v_lds + ((j - 1) & 1) * VP;
-    pw_fast_step<NT, true>(t, s_pend, p_pend, kb, vb, kl, vl, vl_last, 0, g, scale_log2, next, wave);
-    pw_fast_step<NT, false>(t, s_pend, p_pend, kb, vb, kl, vl, vl_last, 1, g, scale_log2, next, wave);
+    pw_fast_step<NT, true, BIAS>(t, s_pend, p_pend, kb, vb, kl, vl, vl_last, 0, g, scale_log2, next, wave, 64 * j);
+    pw_fast_step<NT, false, BIAS>(t, s_pend, p_pend, kb, vb, kl, vl, vl_last, 1, g, scale_log2, next, wave, 64 * j + 32);
     // asked for here, not earlier: scalar loads count with the LDS reads, and a wait for an LDS read
     // that follows one would wait for all of them; the barrier below waits for everything anyway
     __builtin_amdgcn_sched_barrier(0);
@@ -492,7 +506,7 @@ attention_prefill_wide_kernel(
   for (; j <= pbB + 1; ++j) {
     if (j + 1 <= pbB) pw_stage<Pw<NT>::K_CHUNKS>(k_base + ((j + 1) & 1) * KP * 16, pw_page(kp, pt[j + 1], num_pages, k_stride, lane), wave);
     if (j <= pbB) pw_stage<Pw<NT>::V_CHUNKS>(v_base + (j & 1) * VP * 16, pw_page(vp, pt[j], num_pages, v_stride, lane), wave);
-    pw_plain_epoch<NT>(t, s_pend, p_pend, j, hsA, hsB, k_lds + (j & 1) * KP, v_lds + ((j - 1) & 1) * VP, kl, vl,
+    pw_plain_epoch<NT, BIAS>(t, s_pend, p_pend, j, hsA, hsB, k_lds + (j & 1) * KP, v_lds + ((j - 1) & 1) * VP, kl, vl,
                        vl_last, g, scale_log2);
     pw_epoch_end();
   }
@@ -544,18 +558,22 @@ int he_attention_prefill_wide(void* out, const void* q, const void* kpool, const
   HE_REQUIRE(gx * H * num_seqs < (1ll << 31), "he_attention_prefill_wide: grid too large");
   dim3 grid((unsigned)gx, H, num_seqs);
   hipStream_t s = (hipStream_t)stream;
+#define PREFILL_WIDE_ARGS                                                                      \
+  (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,           \
+      (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,          \
+      (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale, parts, ws_o, ws_ml, ex
 #define PREFILL_WIDE(NTV)                                                                       \
   case NTV:                                                                                     \
-    attention_prefill_wide_kernel<NTV><<<grid, 64 * PW_WAVES, 0, s>>>(                          \
-        (uint16_t*)out, (const uint16_t*)q, (const uint16_t*)kpool, (const uint16_t*)vpool,     \
-        (const int32_t*)cu_seqlens, (const int32_t*)seq_slot, (const int32_t*)seq_start,        \
-        (const int32_t*)page_table, max_blocks, num_pages, H, KVH, window, scale, parts, ws_o,  \
-        ws_ml, ex);                                                                             \
+    if (ex.slopes != nullptr)                                                                   \
+      attention_prefill_wide_kernel<NTV, true><<<grid, 64 * PW_WAVES, 0, s>>>(PREFILL_WIDE_ARGS);  \
+    else                                                                                        \
+      attention_prefill_wide_kernel<NTV, false><<<grid, 64 * PW_WAVES, 0, s>>>(PREFILL_WIDE_ARGS); \
     break;
   switch (hd / 16) {
     PREFILL_WIDE(1) PREFILL_WIDE(2) PREFILL_WIDE(3) PREFILL_WIDE(4)
     PREFILL_WIDE(5) PREFILL_WIDE(6) PREFILL_WIDE(7) PREFILL_WIDE(8)
   }
 #undef PREFILL_WIDE
+#undef PREFILL_WIDE_ARGS
   return he_check_launch("he_attention_prefill_wide");
 }

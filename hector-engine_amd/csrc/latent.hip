@@ -69,75 +69,18 @@ __global__ __launch_bounds__(256) void head_product_kernel(T* __restrict__ out, 
     if (r0 + r < rows) out[(r0 + r) * o_row + h * o_head + n] = from_float<T>(total[r]);
 }
 
-// The same sums in the same order for a step of many rows: a workgroup takes 4 x HP_ROWS rows (a wavefront each
-// HP_ROWS of them) of one head and 64 neighbouring n; a lane forms the four quarter sums of a chunk one after the
-// other and adds them as the kernel above does, so a row has the same bits whichever kernel ran it.
-template <typename T, typename TW>
-__global__ __launch_bounds__(256) void head_product_rows_kernel(T* __restrict__ out, int64_t o_row, int64_t o_head,
-                                                                const T* __restrict__ x, int64_t x_row, int64_t x_head,
-                                                                const TW* __restrict__ w, int rows, int K, int N) {
-  __shared__ float xs[4 * HP_ROWS][HP_KCHUNK];
-  const int h = blockIdx.y;
-  const int64_t b0 = (int64_t)blockIdx.z * 4 * HP_ROWS;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = blockIdx.x * 64 + lane;
-  const int nc = min(n, N - 1);
-  const TW* wh = w + (int64_t)h * K * N;
-  float total[HP_ROWS];
-#pragma unroll
-  for (int r = 0; r < HP_ROWS; ++r) total[r] = 0.f;
-  for (int k0 = 0; k0 < K; k0 += HP_KCHUNK) {
-    const int kc = min(HP_KCHUNK, K - k0);
-    __syncthreads();
-    for (int i = threadIdx.x; i < 4 * HP_ROWS * kc; i += blockDim.x) {
-      const int r = i / kc, k = i % kc;
-      xs[r][k] = b0 + r < rows ? to_float(x[(b0 + r) * x_row + h * x_head + k0 + k]) : 0.f;
-    }
-    __syncthreads();
-    const int per = (kc + 3) / 4;
-    float quarter[4][HP_ROWS];
-#pragma unroll
-    for (int part = 0; part < 4; ++part) {
-      const int ka = part * per, kb = min(kc, ka + per);
-#pragma unroll
-      for (int r = 0; r < HP_ROWS; ++r) quarter[part][r] = 0.f;
-      // a plain loop: with many rows the other wavefronts hide a load's way (eight loads at a time were slower here)
-      for (int k = ka; k < kb; ++k) {
-        const float wv = to_float(wh[(int64_t)(k0 + k) * N + nc]);
-#pragma unroll
-        for (int r = 0; r < HP_ROWS; ++r) quarter[part][r] = fmaf(xs[wave * HP_ROWS + r][k], wv, quarter[part][r]);
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < HP_ROWS; ++r)
-      total[r] += ((quarter[0][r] + quarter[1][r]) + quarter[2][r]) + quarter[3][r];
-  }
-  if (n >= N) return;
-#pragma unroll
-  for (int r = 0; r < HP_ROWS; ++r) {
-    const int64_t row = b0 + wave * HP_ROWS + r;
-    if (row < rows) out[row * o_row + h * o_head + n] = from_float<T>(total[r]);
-  }
-}
-
 extern "C" int he_head_product(void* out, int64_t o_row, int64_t o_head, const void* x, int64_t x_row, int64_t x_head,
                                const void* w, int w_dtype, int rows, int H, int K, int N, int dtype, void* stream) {
   HE_REQUIRE(rows >= 0 && H > 0 && K > 0 && N > 0 && H <= 65535, "he_head_product: bad sizes H=%d K=%d N=%d", H, K, N);
   HE_REQUIRE((dtype == HE_BF16 || dtype == HE_F32) && (w_dtype == HE_BF16 || w_dtype == HE_F32), "he_head_product: unknown dtype");
   if (rows == 0) return 0;
   const int threads = 256;
-  const bool many = rows > 4 * HP_ROWS;      // a step of many rows: a wavefront takes whole rows, not a quarter of the k
-  const int per_group = many ? 4 * HP_ROWS : HP_ROWS;
-  const dim3 grid((N + 63) / 64, H, (rows + per_group - 1) / per_group);
+  const dim3 grid((N + 63) / 64, H, (rows + HP_ROWS - 1) / HP_ROWS);
   HE_REQUIRE(grid.z <= 65535, "he_head_product: %d rows are too many for one launch", rows);
   hipStream_t s = (hipStream_t)stream;
-#define HP_LAUNCH(T, TW)                                                                                              \
-  if (many)                                                                                                           \
-    head_product_rows_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head,      \
-                                                             (const TW*)w, rows, K, N);                               \
-  else                                                                                                                \
-    head_product_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head,           \
-                                                        (const TW*)w, rows, K, N)
+#define HP_LAUNCH(T, TW)                                                                                    \
+  head_product_kernel<T, TW><<<grid, threads, 0, s>>>((T*)out, o_row, o_head, (const T*)x, x_row, x_head, \
+                                                      (const TW*)w, rows, K, N)
   if (dtype == HE_BF16 && w_dtype == HE_BF16) {
     HP_LAUNCH(bf16_t, bf16_t);
   } else if (dtype == HE_BF16) {

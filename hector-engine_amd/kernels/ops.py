@@ -1229,8 +1229,7 @@ def attention_prefill(out, q, kpool, vpool, cu_seqlens, seq_slot, seq_start, pag
     name it: 16 queries a wavefront with operands from global memory, or 32 queries a
     wavefront with the pages shared through LDS (head sizes up to 128). parts > 1 (kernel 2):
     the keys in that many parts side by side, joined by a second launch; the workspace holds
-    attention_prefill_workspace_floats() floats. chunk, sinks, gate, slopes: as attention_plain takes them
-    (with slopes the library's choice is kernel 1 and the keys stay in one part)."""
+    attention_prefill_workspace_floats() floats. chunk, sinks, gate, slopes: as attention_plain takes them."""
     _check_attention(out, q, kpool, vpool, page_table, total_rows, H, KVH, hd)
     _need(q, "q", torch.bfloat16)
     gate_ptr, gate_stride = _gate_view(gate, q, total_rows, H)

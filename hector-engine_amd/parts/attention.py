@@ -452,8 +452,7 @@ class Attention(Mixer):
             most = min(most, self.window + ctx.max_q_len)
         if self.chunk > 0:
             most = min(most, self.chunk + ctx.max_q_len)
-        # (the kernel that takes distance slopes walks a query's keys in one part)
-        parts = 1 if self.slopes is not None else ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
+        parts = ops.attention_prefill_parts(ctx.num_seqs, ctx.max_q_len, H, hd, most)
         ws = ctx.alloc((ops.attention_prefill_workspace_floats(rows, H, hd, parts),), torch.float32) \
             if parts > 1 else None
         if ctx.padded:

@@ -293,7 +293,8 @@ def test_weights_that_are_the_softmax_over_the_chosen_logits(ops, E, top):
 
 
 # ------------------------------------------------------------------ attention with distance slopes
-@pytest.mark.parametrize("kind,dtype", [("plain", "float32"), ("plain", "bfloat16"), ("decode", "bfloat16"), ("prefill", "bfloat16")])
+@pytest.mark.parametrize("kind,dtype", [("plain", "float32"), ("plain", "bfloat16"), ("decode", "bfloat16"), ("prefill", "bfloat16"),
+                                        ("prefill_without_lds", "bfloat16"), ("prefill_in_parts", "bfloat16")])
 @pytest.mark.parametrize("H,KVH,hd", [(6, 2, 32), (4, 1, 96), (3, 3, 16), (20, 1, 48), (2, 1, 160)])
 def test_scores_that_fall_with_the_distance(ops, kind, dtype, H, KVH, hd):
     """Every attention kernel with a slope a head, against the direct sums: prompts, a continuation and single tokens
@@ -330,9 +331,17 @@ def test_scores_that_fall_with_the_distance(ops, kind, dtype, H, KVH, hd):
         ws = torch.empty(ops.attention_decode_workspace_floats(rows, H, KVH, hd, 4096), device="cuda")
         ops.attention_decode(out, dev(q), *pools, dev(positions), dev(row_seq), i32(slots), dev(table), rows, H, KVH, hd, 0,
                              scale, 4096, ws, slopes=dev(slopes))
-    else:
+    elif kind == "prefill_in_parts":
+        if hd > 128:
+            pytest.skip("keys in parts are for head sizes up to 128")
+        ws = torch.empty(ops.attention_prefill_workspace_floats(rows, H, hd, 3), device="cuda")
         ops.attention_prefill(out, dev(q), *pools, cu, i32(slots), starts, dev(table), len(lengths), max(q_lens), rows, H, KVH,
-                              hd, 0, scale, slopes=dev(slopes))
+                              hd, 0, scale, kernel=2, parts=3, workspace=ws, slopes=dev(slopes))
+    else:
+        # the library's choice (32 queries a wavefront with pages shared through LDS up to a head size of 128), or
+        # the kernel of 16 queries a wavefront named outright
+        ops.attention_prefill(out, dev(q), *pools, cu, i32(slots), starts, dev(table), len(lengths), max(q_lens), rows, H, KVH,
+                              hd, 0, scale, kernel=1 if kind == "prefill_without_lds" else 0, slopes=dev(slopes))
     r, moved = 0, 0.0
     for i, (n, m) in enumerate(zip(lengths, q_lens)):
         want = P.distance_attention(qs[i].double(), ks[i].double(), vs[i].double(), scale, slopes.double().tolist(), n - m)
