@@ -55,8 +55,8 @@ def softplus(z):
 
 
 def short_conv(u, taps, before=None):
-    """u [T, C], taps [C, K]: y_t = sum_j taps[:, j] u_(t - K + 1 + j), zeros (or the rows of
-    `before`, the K - 1 inputs ahead of u) in front of the sequence."""
+    """u [T, C], taps [C, K]: y[t] = sum over j < K of taps[:, j] * u[t - (K - 1 - j)] (the last column weighs
+    the row's own input), with zeros (or the rows of `before`, the K - 1 inputs ahead of u) in front of the sequence."""
     T, C = u.shape
     K = taps.shape[1]
     front = torch.zeros((K - 1, C), dtype=u.dtype) if before is None else before
