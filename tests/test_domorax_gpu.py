@@ -87,7 +87,7 @@ def plain_delta(x, ba, a_log, dt_bias, H, G, d, e, q_scale):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,d,e", [(4, 2, 16, 24), (3, 3, 8, 8), (2, 1, 40, 12), (6, 2, 5, 7), (1, 1, 1, 1), (2, 2, 130, 3),
-                                     (2, 1, 96, 64), (1, 1, 32, 70)])
+                                     (2, 1, 96, 64), (1, 1, 32, 70), (1, 1, 300, 5)])
 def test_delta_rule_in_portions_and_batches_equals_the_whole(ops, dtype, H, G, d, e):
     tdt = TORCH[dtype]
     wide = 2 * G * d + H * e + 8                                  # q | k | v inside wider rows, as behind a convolution
